@@ -24,7 +24,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from .needs import PagedKvNeed, StateNeed
+from .needs import JointNeed, PagedKvNeed, StateNeed, paged_need, state_need
 from .pages import OutOfPages, PagePool
 from .prefix import PrefixIndex
 
@@ -177,7 +177,7 @@ class PageGroup:
 
 
 class CacheManager:
-    """`needs[i]` is the need of run-order entry i (PagedKvNeed, StateNeed or None); `reads_from[i]`
+    """`needs[i]` is the need of run-order entry i (PagedKvNeed, StateNeed, a JointNeed of both, or None); `reads_from[i]`
     is the entry whose pages entry i reads instead of keeping its own (or None)."""
 
     def __init__(self, needs: Sequence, reads_from: Sequence[Optional[int]], *, page_size: int, n_pages: int, max_requests: int,
@@ -195,14 +195,13 @@ class CacheManager:
                 if needs[src] != need or not isinstance(need, PagedKvNeed):
                     raise CacheError(f"run-order entry {i} reads the cache of entry {src}, whose need differs: {needs[src]} against {need}")
                 continue
-            if isinstance(need, PagedKvNeed):
-                by_need.setdefault(need, []).append(i)
-            elif isinstance(need, StateNeed):
-                if allocate_storage:
-                    self.states[i] = torch.zeros((max_requests + 1, *need.shape), dtype=need.dtype, device=device)
-            elif need is not None:
+            if need is not None and not isinstance(need, (PagedKvNeed, StateNeed, JointNeed)):
                 raise CacheError(f"run-order entry {i} has an unknown cache need {need!r}")
-        self._state_needed = any(isinstance(need, StateNeed) for need in needs)
+            if paged_need(need) is not None:
+                by_need.setdefault(paged_need(need), []).append(i)
+            if state_need(need) is not None and allocate_storage:
+                self.states[i] = torch.zeros((max_requests + 1, *state_need(need).shape), dtype=state_need(need).dtype, device=device)
+        self._state_needed = any(state_need(need) is not None for need in needs)
         for need, entries in by_need.items():
             g = PageGroup(need, entries, n_pages, page_size, max_requests, max_positions, dtype, device, allocate_storage)
             for li, e in enumerate(entries):

@@ -40,3 +40,25 @@ class StateNeed:
     """A state of fixed size per request (for instance a recurrent state), zeroed when a request starts."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+
+@dataclass(frozen=True)
+class JointNeed:
+    """What a mixer made of several mixers asks for one run-order entry: pages and a fixed-size state side by side (at most one
+    of each; either may be absent)."""
+    paged: Optional[PagedKvNeed] = None
+    state: Optional[StateNeed] = None
+
+
+def paged_need(need) -> Optional[PagedKvNeed]:
+    """The pages an entry's need asks for, or None."""
+    if isinstance(need, JointNeed):
+        return need.paged
+    return need if isinstance(need, PagedKvNeed) else None
+
+
+def state_need(need) -> Optional[StateNeed]:
+    """The fixed-size state an entry's need asks for, or None."""
+    if isinstance(need, JointNeed):
+        return need.state
+    return need if isinstance(need, StateNeed) else None

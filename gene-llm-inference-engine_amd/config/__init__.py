@@ -1,9 +1,11 @@
 """Typed configurations, the architecture registry and the neutral model description."""
 from .spec import (AttentionSpec, DenseMlpSpec, GatedDeltaSpec, InterleavedRotarySpec, LatentAttentionSpec, LayerSpec, MlstmSpec, ModelSpec,
-                   PartialRotarySpec, RmsNormSpec, RotarySpec, RunEntry, ScaleSpec, SoftCapSpec, SwiGluSpec)
+                   PartialRotarySpec, RejoinSpec, RmsNormSpec, RotarySpec, RoutedExpertsSpec, RunEntry, ScaleSpec, SelectiveScanSpec, SideBySideSpec, SoftCapSpec,
+                   SwiGluSpec, TokenSideInputSpec)
 from .errors import ConfigError
 from .registry import (config_class_for, parse_config, read_config, register_architecture,
                        registered_architectures)
 from .llama import Llama3Scaling, LlamaConfig          # registers itself
 from .fekorax import FekoraxConfig                     # registers itself
 from .rigalorn import RigalornConfig                   # registers itself
+from .zidevik import ZidevikConfig                     # registers itself

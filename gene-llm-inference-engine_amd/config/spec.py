@@ -109,6 +109,9 @@ class AttentionSpec:
     # number in its tensor `value_blend` and v_first the first layer's values of the same row.
     value_family: Optional[str] = None
     value_blend: Optional[str] = None
+    # Every query and key head divided by its root mean square over the head (eps `qk_norm_eps` inside the root), without weights and
+    # behind the rotation (q_norm and k_norm must then be absent).
+    qk_unit_rms: bool = False
 
 
 @dataclass(frozen=True)
@@ -198,6 +201,104 @@ class GatedDeltaSpec:
 
 
 @dataclass(frozen=True)
+class SelectiveScanSpec:
+    """A selective scan (the Mamba recurrence).  `in_proj` [2 inner, hidden] gives [x | z].  x passes a causal convolution per channel
+    (`conv` [inner, conv_taps], the last tap the token's own, bias `conv_bias`, zeros before a sequence's start) and SiLU.  `x_proj`
+    [dt_rank + 2 state, inner] of that gives [dt | B | C]; dt <- softplus(`dt_proj` [inner, dt_rank] dt + `dt_bias`), one step size per
+    channel; A = -exp(`a_log`) [inner, state].  Per channel c and state n, S zero at a sequence's start:
+        S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n        y_c = sum_n S[c, n] C_n + D_c x_c
+    and the mixer's result is `o_proj` (y * SiLU(z)).  A request's state is S and the convolution's last conv_taps - 1 inputs."""
+    kind: ClassVar[str] = "selective_scan"
+    hidden_size: int
+    inner: int
+    state: int
+    dt_rank: int
+    conv_taps: int
+    in_proj: str
+    conv: str
+    conv_bias: str
+    x_proj: str
+    dt_proj: str
+    dt_bias: str
+    a_log: str
+    d_skip: str
+    o_proj: str
+
+
+@dataclass(frozen=True)
+class SideBySideSpec:
+    """Several mixers that read the same rows; the layer's mixer output is sum_i weights[i] * members[i](h).  Each member keeps the
+    cache or state it would keep alone."""
+    kind: ClassVar[str] = "side_by_side"
+    hidden_size: int
+    members: Tuple[Any, ...]
+    weights: Tuple[float, ...]
+
+    def __post_init__(self):
+        if not self.members or len(self.members) != len(self.weights):
+            raise ValueError("mixers side by side: one weight per member, and at least one member")
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """A mixture of gated feed-forwards: `router` [experts, hidden] gives a logit per expert in 32-bit; the scores are their sigmoids
+    (`score` = "sigmoid") or a softmax over all experts ("softmax"); the `top` experts with the largest scores serve the row.  The
+    chosen scores, divided by their sum if `renormalize`, weigh each chosen expert's input (`weigh` = "input": the sum of
+    expert(w h)) or its output ("output": the sum of w expert(h)).  An expert is down(act(gate(a)) * up(a)) without biases.  `shared`,
+    a feed-forward spec of any kind, serves every row and is added."""
+    kind: ClassVar[str] = "routed_experts"
+    hidden_size: int
+    intermediate_size: int
+    n_experts: int
+    top: int
+    router: str
+    gate_projs: Tuple[str, ...]
+    up_projs: Tuple[str, ...]
+    down_projs: Tuple[str, ...]
+    score: str = "sigmoid"
+    renormalize: bool = False
+    weigh: str = "input"
+    activation: str = "silu"
+    shared: Optional[Any] = None
+
+    def __post_init__(self):
+        if not (len(self.gate_projs) == len(self.up_projs) == len(self.down_projs) == self.n_experts) or not 1 <= self.top <= self.n_experts:
+            raise ValueError("routed experts: three matrices per expert, and 1 <= top <= experts")
+
+
+@dataclass(frozen=True)
+class TokenSideInputSpec:
+    """A second input from the token itself, added to the residual stream x behind a layer: with e the columns
+    [first_column, first_column + dim) of the token's row of `table` [vocab, table_width],
+        g = act(`gate_proj` x) * e;   y = `out_proj` g;   x <- x + norm(y)
+    gate_proj [dim, hidden], out_proj [hidden, dim], `norm` a norm spec over hidden."""
+    kind: ClassVar[str] = "token_side_input"
+    hidden_size: int
+    vocab_size: int
+    dim: int
+    table: str
+    table_width: int
+    first_column: int
+    gate_proj: str
+    out_proj: str
+    norm: Any
+    activation: str = "gelu_tanh"
+
+
+@dataclass(frozen=True)
+class RejoinSpec:
+    """The residual stream mixed with the token rows again: x <- `weight` [x; x0] + row `row` of `offsets`, with x0 the rows of the
+    token table as the first layer got them, weight [hidden, 2 hidden] (x's columns first), offsets [rows, hidden] (None: nothing
+    added)."""
+    kind: ClassVar[str] = "rejoin"
+    hidden_size: int
+    weight: str
+    offsets: Optional[str] = None
+    offsets_rows: int = 0
+    row: int = 0
+
+
+@dataclass(frozen=True)
 class MlstmSpec:
     """A matrix memory per head (the mLSTM of xLSTM) with exponential gating kept stable by a running maximum:
         m_t = max(f_t + m_(t-1), i_t)
@@ -249,15 +350,18 @@ class LayerSpec:
     block: str = "prenorm"
     mixer_post_norm: Any = None      # "sandwich" blocks: a norm on what each half puts out, before it joins the residual stream
     feed_forward_post_norm: Any = None
+    after: Tuple[Any, ...] = ()      # specs of parts that change the residual stream in place behind the block, in order (stream parts)
 
 
 @dataclass(frozen=True)
 class RunEntry:
     """One position of the run order.  `layer` indexes `ModelSpec.layers` (a layer may be named by
     several entries).  `cache_of` is None when the entry keeps a cache of its own, or the index of
-    an earlier entry whose cache it reads without writing."""
+    an earlier entry whose cache it reads without writing.  Entries that name one layer share its weights and keep a cache
+    each."""
     layer: int
     cache_of: Optional[int] = None
+    before: Optional[Any] = None     # spec of a part that changes the residual stream in place before this entry's layer runs (a stream part)
 
 
 @dataclass(frozen=True)

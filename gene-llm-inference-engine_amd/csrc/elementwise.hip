@@ -416,7 +416,11 @@ GI_API int gi_rmsnorm_add(const float* y, const void* w, int w_dtype, float* x, 
 // Values may be blended with those another layer made of the same rows: with `v_other` [n_rows, ld_other] and `v_blend` (one
 // number on the device), v <- (1 - blend) v + blend v_other is what goes into the page; `v_keep` [n_rows, ld_keep], if given, gets
 // this layer's values (with their bias, before any blending) for such a reader.
+// `flags`: NRS_NEIGHBOURS turns the pairs (2i, 2i + 1), i < rot/2, instead (angle i for pair i); NRS_UNIT_RMS divides every query and
+// key head by its root mean square without weights (q_norm and k_norm must then be absent); NRS_NORM_LAST takes the norm, of
+// either form, behind the rotation instead of in front of it.
 constexpr int NRS_MAX_HD = 512;
+constexpr int NRS_NEIGHBOURS = 1, NRS_UNIT_RMS = 2, NRS_NORM_LAST = 4;
 
 template <typename TQ, typename TC, typename TW>
 __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
@@ -427,7 +431,7 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
                                                             int page_size, int n_heads, int n_kv, int hd, int vd,
                                                             const float* __restrict__ q_bias, const float* __restrict__ k_bias,
                                                             const float* __restrict__ v_bias, const float* __restrict__ v_other, long ld_other,
-                                                            const float* __restrict__ v_blend, float* __restrict__ v_keep, long ld_keep) {
+                                                            const float* __restrict__ v_blend, float* __restrict__ v_keep, long ld_keep, int flags) {
     __shared__ float s[NRS_MAX_HD];
     const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
@@ -456,13 +460,14 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
         s[d] = x;
         ss = fmaf(x, x, ss);
     }
-    if (w != nullptr) {
-        const float r = 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps);
-        for (int d = lane; d < hd; d += 64) s[d] = load_f32(w, d) * (r * s[d]);
+    const bool normed = w != nullptr || (flags & NRS_UNIT_RMS), norm_last = normed && (flags & NRS_NORM_LAST);
+    const float r = normed ? 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps) : 1.0f;      // (a rotation keeps the sum of squares: the same number in front of it and behind it)
+    if (normed && !norm_last) {
+        for (int d = lane; d < hd; d += 64) s[d] = w != nullptr ? load_f32(w, d) * (r * s[d]) : r * s[d];
     }
     __syncthreads();
     const int half = rot / 2;
-    const bool turn = cos_t != nullptr && rot > 0;
+    const bool turn = cos_t != nullptr && rot > 0, neighbours = flags & NRS_NEIGHBOURS;
     TC* kdst = nullptr;
     TQ* qdst = nullptr;
     if (is_q) qdst = q_out + ((size_t)t * n_heads + h) * hd;
@@ -473,10 +478,16 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
     for (int d = lane; d < hd; d += 64) {
         float out = s[d];
         if (turn && d < rot) {
-            const int i = d < half ? d : d - half;
-            const float c = cos_t[(size_t)t * half + i], sn = sin_t[(size_t)t * half + i];
-            out = d < half ? s[d] * c - s[d + half] * sn : s[d] * c + s[d - half] * sn;
+            if (neighbours) {
+                const float c = cos_t[(size_t)t * half + d / 2], sn = sin_t[(size_t)t * half + d / 2];
+                out = (d & 1) ? s[d] * c + s[d - 1] * sn : s[d] * c - s[d + 1] * sn;
+            } else {
+                const int i = d < half ? d : d - half;
+                const float c = cos_t[(size_t)t * half + i], sn = sin_t[(size_t)t * half + i];
+                out = d < half ? s[d] * c - s[d + half] * sn : s[d] * c + s[d - half] * sn;
+            }
         }
+        if (norm_last) out = w != nullptr ? load_f32(w, d) * (r * out) : r * out;
         if (is_q) store_f32(qdst, d, out); else store_f32(kdst, d, out);
     }
 }
@@ -486,7 +497,9 @@ GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, lo
                               const int* table, int table_stride, void* q_out, int q_dtype, void* cache, int cache_dtype, long page_stride,
                               int page_size, int n_rows, int n_heads, int n_kv, int hd, int vd, const float* q_bias, const float* k_bias,
                               const float* v_bias, const float* v_other, long ld_other, const float* v_blend, float* v_keep, long ld_keep,
-                              hipStream_t stream) {
+                              int flags, hipStream_t stream) {
+    GI_REQUIRE(!(flags & NRS_UNIT_RMS) || (q_norm == nullptr && k_norm == nullptr), "norm_rope_store: heads divided by their root mean square have no norm weights");
+    GI_REQUIRE(!(flags & NRS_NEIGHBOURS) || rot % 2 == 0, "norm_rope_store: neighbouring pairs need an even number of turned channels");
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && hd > 0 && hd <= NRS_MAX_HD && vd > 0, "norm_rope_store: bad sizes (rows %d heads %d kv %d hd %d vd %d)",
                n_rows, n_heads, n_kv, hd, vd);
     GI_REQUIRE((v_other == nullptr || (v_blend != nullptr && ld_other >= (long)n_kv * vd)) && (v_keep == nullptr || ld_keep >= (long)n_kv * vd) &&
@@ -500,7 +513,7 @@ GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, lo
 #define LAUNCH(TQ, TC, TW)                                                                                                                    \
     norm_rope_store_kernel<TQ, TC, TW><<<grid, 64, 0, stream>>>(q, k, v, ldq, ldk, ldv, (const TW*)q_norm, (const TW*)k_norm, eps, cos_t, sin_t, rot, pos, \
                                                                 slot, table, table_stride, (TQ*)q_out, (TC*)cache, page_stride, page_size, n_heads, n_kv, hd, vd, \
-                                                                q_bias, k_bias, v_bias, v_other, ld_other, v_blend, v_keep, ld_keep)
+                                                                q_bias, k_bias, v_bias, v_other, ld_other, v_blend, v_keep, ld_keep, flags)
     if (q_dtype == GI_F32 && cache_dtype == GI_F32 && norm_dtype == GI_F32) LAUNCH(float, float, float);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_F32) LAUNCH(bf16_t, bf16_t, float);
@@ -608,5 +621,95 @@ GI_API int gi_rmsnorm_add_norm(const float* y, const void* w, const void* w_next
     else return gi_fail("rmsnorm_add_norm: unknown dtypes %d, %d", w_dtype, out_dtype);
 #undef LAUNCH
     GI_CHECK_LAUNCH("rmsnorm_add_norm");
+    return 0;
+}
+
+// ------------------------------------------------- rows laid side by side, weighted sums of rows, a vector added to every row
+// out[t] = [a[t]; b[t]] stored as a product reads it (b == nullptr: a alone, which makes it a conversion of rows).
+template <typename TO>
+__global__ __launch_bounds__(256) void concat_rows_kernel(const float* __restrict__ a, long lda, int wa, const float* __restrict__ b, long ldb, int wb,
+                                                         TO* __restrict__ out, long ldo) {
+    const size_t t = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < wa) store_f32(out + t * ldo, c, a[t * lda + c]);
+    else if (c < wa + wb) store_f32(out + t * ldo, c, b[t * ldb + (c - wa)]);
+}
+
+GI_API int gi_concat_rows(const float* a, long lda, int wa, const float* b, long ldb, int wb, void* out, int out_dtype, long ldo, int n_rows, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && wa > 0 && wb >= 0 && lda >= wa && (b == nullptr ? wb == 0 : ldb >= wb) && ldo >= wa + wb, "concat_rows: bad sizes (rows %d, %d + %d columns)", n_rows, wa, wb);
+    dim3 grid(n_rows, (wa + wb + 255) / 256);
+    GI_REQUIRE(grid.y <= 65535, "concat_rows: rows too long");
+    if (out_dtype == GI_F32) concat_rows_kernel<float><<<grid, 256, 0, stream>>>(a, lda, wa, b, ldb, wb, (float*)out, ldo);
+    else if (out_dtype == GI_BF16) concat_rows_kernel<bf16_t><<<grid, 256, 0, stream>>>(a, lda, wa, b, ldb, wb, (bf16_t*)out, ldo);
+    else return gi_fail("concat_rows: unknown dtype %d", out_dtype);
+    GI_CHECK_LAUNCH("concat_rows");
+    return 0;
+}
+
+// x[t] += sa * a[t] + sb * b[t]  (b == nullptr: the first term alone); the two terms are added to each other first.
+__global__ __launch_bounds__(256) void add_weighted_kernel(float* __restrict__ x, long ldx, const float* __restrict__ a, long lda, float sa,
+                                                          const float* __restrict__ b, long ldb, float sb, int dim) {
+    const size_t t = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= dim) return;
+    float y = sa * a[t * lda + c];
+    if (b != nullptr) y = fmaf(sb, b[t * ldb + c], y);
+    x[t * ldx + c] += y;
+}
+
+GI_API int gi_add_weighted(float* x, long ldx, const float* a, long lda, float sa, const float* b, long ldb, float sb, int n_rows, int dim, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && ldx >= dim && lda >= dim && (b == nullptr || ldb >= dim), "add_weighted: bad sizes (rows %d, dim %d)", n_rows, dim);
+    dim3 grid(n_rows, (dim + 255) / 256);
+    GI_REQUIRE(grid.y <= 65535, "add_weighted: rows too long");
+    add_weighted_kernel<<<grid, 256, 0, stream>>>(x, ldx, a, lda, sa, b, ldb, sb, dim);
+    GI_CHECK_LAUNCH("add_weighted");
+    return 0;
+}
+
+// x[t] += v for every row t.
+template <typename TV>
+__global__ __launch_bounds__(256) void add_vector_kernel(float* __restrict__ x, long ldx, const TV* __restrict__ v, int dim) {
+    const size_t t = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c < dim) x[t * ldx + c] += load_f32(v, c);
+}
+
+GI_API int gi_add_vector(float* x, long ldx, const void* v, int v_dtype, int n_rows, int dim, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && ldx >= dim, "add_vector: bad sizes (rows %d, dim %d)", n_rows, dim);
+    dim3 grid(n_rows, (dim + 255) / 256);
+    GI_REQUIRE(grid.y <= 65535, "add_vector: rows too long");
+    if (v_dtype == GI_F32) add_vector_kernel<float><<<grid, 256, 0, stream>>>(x, ldx, (const float*)v, dim);
+    else if (v_dtype == GI_BF16) add_vector_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, ldx, (const bf16_t*)v, dim);
+    else return gi_fail("add_vector: unknown dtype %d", v_dtype);
+    GI_CHECK_LAUNCH("add_vector");
+    return 0;
+}
+
+// out[t, c] = act(u[t, c]) * table[tokens[t], first + c]: a gate on columns of the token's own row of a table.  act: 0 SiLU, 1 the tanh
+// form of GELU.
+template <typename TT, typename TO>
+__global__ __launch_bounds__(64) void gate_token_columns_kernel(const float* __restrict__ u, long ldu, const TT* __restrict__ table, long ldt, int first,
+                                                               const int* __restrict__ tokens, TO* __restrict__ out, long ldo, int dim, int act) {
+    const size_t t = blockIdx.x;
+    const TT* row = table + (size_t)tokens[t] * ldt + first;
+    for (int c = threadIdx.x; c < dim; c += 64) {
+        const float z = u[t * ldu + c];
+        const float a = act == 1 ? 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))) : z / (1.0f + expf(-z));
+        store_f32(out + t * ldo, c, a * load_f32(row, c));
+    }
+}
+
+GI_API int gi_gate_token_columns(const float* u, long ldu, const void* table, int table_dtype, long ldt, int first, const int* tokens, void* out, int out_dtype,
+                                 long ldo, int n_rows, int dim, int act, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && ldu >= dim && ldo >= dim && first >= 0 && ldt >= first + dim && (act == 0 || act == 1),
+               "gate_token_columns: bad sizes (rows %d, dim %d, columns from %d of %ld)", n_rows, dim, first, ldt);
+#define LAUNCH(TT, TO) gate_token_columns_kernel<TT, TO><<<n_rows, 64, 0, stream>>>(u, ldu, (const TT*)table, ldt, first, tokens, (TO*)out, ldo, dim, act)
+    if (table_dtype == GI_F32 && out_dtype == GI_F32) LAUNCH(float, float);
+    else if (table_dtype == GI_BF16 && out_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (table_dtype == GI_BF16 && out_dtype == GI_F32) LAUNCH(bf16_t, float);
+    else if (table_dtype == GI_F32 && out_dtype == GI_BF16) LAUNCH(float, bf16_t);
+    else return gi_fail("gate_token_columns: unknown dtypes %d, %d", table_dtype, out_dtype);
+#undef LAUNCH
+    GI_CHECK_LAUNCH("gate_token_columns");
     return 0;
 }

@@ -1,0 +1,203 @@
+// The selective scan (a state-space recurrence whose step size and in/out vectors depend on the token), stepped token by token in
+// 32-bit.  Per channel c and state n of a request:
+//     S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n        y_c = sum_n S[c, n] C_n + D_c x_c
+// with A = -exp(A_log) [channels, states], dt_c = softplus(pre_c + bias_c) one per channel and token, B and C [states] one per
+// token.  x is the channel's input behind a short causal convolution (taps [channels, taps], the last tap the token's own, a bias)
+// and SiLU; the read-out is multiplied by SiLU of a gate z.  Channels never meet, so a wave owns 16 of them for one request of the
+// step and walks the request's rows in order; a channel's states lie over four neighbouring lanes (state n with lane n mod 4),
+// whose shares of the read-out's sum are added by lane moves in an order that the number of states alone fixes: a request's
+// results have the same bits however its rows are cut into steps.  A token's inputs are asked for while the token before it is
+// worked on.
+//
+// State of one request slot, 32-bit: S [channels][states], then the convolution's last taps - 1 inputs [taps - 1][channels].
+#include "common.h"
+
+namespace {
+
+constexpr int SSM_MAX_TAPS = 8;
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// How many of the rows t-1, t-2, ... (at most `most`) belong to the same request as row t and directly precede it.
+__device__ __forceinline__ int rows_before(const int* __restrict__ slot, const int* __restrict__ pos, int t, int most) {
+    int n = 0;
+    while (n < most && t - n - 1 >= 0 && slot[t - n - 1] == slot[t] && pos[t - n - 1] == pos[t] - n - 1) ++n;
+    return n;
+}
+
+// Convolution + bias + SiLU of one row's channels.  Rows of the same request in this step are read where they lie; what came before
+// the step comes from the request's tail.  `move_tail` (steps of single rows: nobody else reads this request's tail): the thread that
+// read a channel's tail also moves it on.
+template <typename TO>
+__global__ __launch_bounds__(256) void ssm_conv_kernel(const float* __restrict__ pre, long ld, const float* __restrict__ taps, int n_taps,
+                                                      const float* __restrict__ bias, float* __restrict__ tail, long tail_stride, int move_tail,
+                                                      const int* __restrict__ slot, const int* __restrict__ pos, float* __restrict__ x,
+                                                      TO* __restrict__ x_low, int inner) {
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= inner) return;
+    const int before = rows_before(slot, pos, t, n_taps - 1);
+    float* old = tail + (size_t)slot[t] * tail_stride;
+    float y = bias[c];
+    for (int j = 0; j < n_taps; ++j) {
+        const int back = n_taps - 1 - j;                      // rows before t that tap j reads
+        const float v = back <= before ? pre[(size_t)(t - back) * ld + c] : old[(size_t)(n_taps - 1 - (back - before)) * inner + c];
+        y = fmaf(taps[(size_t)c * n_taps + j], v, y);
+    }
+    if (move_tail) {
+        for (int i = 0; i + 2 < n_taps; ++i) old[(size_t)i * inner + c] = old[(size_t)(i + 1) * inner + c];
+        if (n_taps > 1) old[(size_t)(n_taps - 2) * inner + c] = pre[(size_t)t * ld + c];
+    }
+    y = silu_f(y);
+    x[(size_t)t * inner + c] = y;
+    if (x_low != nullptr) store_f32(x_low, (size_t)t * inner + c, y);
+}
+
+// Behind the convolution: every request's tail becomes the last taps - 1 inputs of (its old tail, its rows of this step).
+__global__ __launch_bounds__(256) void ssm_tail_kernel(const float* __restrict__ pre, long ld, int inner, int n_taps, const int* __restrict__ seg_start,
+                                                      const int* __restrict__ seg_len, const int* __restrict__ slot, float* __restrict__ tail,
+                                                      long tail_stride) {
+    const int n = seg_len[blockIdx.x];
+    if (n <= 0) return;
+    const int t0 = seg_start[blockIdx.x], keep = n_taps - 1;
+    float* mine = tail + (size_t)slot[t0] * tail_stride;
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < inner; c += 256 * gridDim.y) {
+        float held[SSM_MAX_TAPS];
+#pragma unroll
+        for (int s = 0; s < SSM_MAX_TAPS; ++s) {
+            if (s >= keep) break;
+            const int e = n - keep + s;                           // row of the step, or (negative) place before it
+            held[s] = e >= 0 ? pre[(size_t)(t0 + e) * ld + c] : mine[(size_t)(keep + e) * inner + c];
+        }
+#pragma unroll
+        for (int s = 0; s < SSM_MAX_TAPS; ++s) {
+            if (s >= keep) break;
+            mine[(size_t)s * inner + c] = held[s];
+        }
+    }
+}
+
+// The recurrence: one wave per (request of the step, 16 channels).  lane = channel * 4 + part; a lane keeps the states part,
+// part + 4, ... of its channel (NPL of them at most).
+template <int NPL, typename TO>
+__global__ __launch_bounds__(64) void ssm_scan_kernel(const float* __restrict__ x, const float* __restrict__ dt_pre, long ld_dt, const float* __restrict__ dt_bias,
+                                                     const float* __restrict__ bc, long ld_bc, int b_off, int c_off, const float* __restrict__ z, long ld_z,
+                                                     const float* __restrict__ a_log, const float* __restrict__ d_skip, const int* __restrict__ seg_start,
+                                                     const int* __restrict__ seg_len, const int* __restrict__ row_slot, float* __restrict__ state,
+                                                     long state_stride, TO* __restrict__ out, long ldo, int inner, int n_state) {
+    const int n_rows = seg_len[blockIdx.x];
+    if (n_rows <= 0) return;
+    const int t0 = seg_start[blockIdx.x], lane = threadIdx.x, part = lane & 3;
+    const int c = blockIdx.y * 16 + (lane >> 2);
+    const bool live = c < inner;
+    const int cc = live ? c : inner - 1;                          // (idle lanes walk along on the last channel and store nothing)
+    float* mine = state + (size_t)row_slot[t0] * state_stride + (size_t)cc * n_state;
+    float S[NPL], A[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+        const int n = part + 4 * i;
+        S[i] = n < n_state ? mine[n] : 0.f;
+        A[i] = n < n_state ? -expf(a_log[(size_t)cc * n_state + n]) : 0.f;
+    }
+    const float bias = dt_bias[cc], skip = d_skip[cc];
+    float xv = x[(size_t)t0 * inner + cc], pre = dt_pre[(size_t)t0 * ld_dt + cc], zv = z[(size_t)t0 * ld_z + cc];
+    float B[NPL], C[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+        const int n = min(part + 4 * i, n_state - 1);
+        B[i] = bc[(size_t)t0 * ld_bc + b_off + n];
+        C[i] = bc[(size_t)t0 * ld_bc + c_off + n];
+    }
+    for (int r = 0; r < n_rows; ++r) {
+        const int t = t0 + r, tn = t0 + min(r + 1, n_rows - 1);      // the next row's inputs are asked for now (the last row asks for itself again)
+        const float nx = x[(size_t)tn * inner + cc], npre = dt_pre[(size_t)tn * ld_dt + cc], nz = z[(size_t)tn * ld_z + cc];
+        float nB[NPL], nC[NPL];
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) {
+            const int n = min(part + 4 * i, n_state - 1);
+            nB[i] = bc[(size_t)tn * ld_bc + b_off + n];
+            nC[i] = bc[(size_t)tn * ld_bc + c_off + n];
+        }
+        const float dt = softplus_f(pre + bias), dx = dt * xv;
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) {
+            if (part + 4 * i < n_state) {
+                S[i] = fmaf(expf(dt * A[i]), S[i], dx * B[i]);
+                acc = fmaf(S[i], C[i], acc);
+            }
+        }
+        acc += __shfl_xor(acc, 1, 64);
+        acc += __shfl_xor(acc, 2, 64);
+        if (live && part == 0) store_f32(out, (size_t)t * ldo + c, fmaf(skip, xv, acc) * silu_f(zv));
+        xv = nx, pre = npre, zv = nz;
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) B[i] = nB[i], C[i] = nC[i];
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) {
+            const int n = part + 4 * i;
+            if (n < n_state) mine[n] = S[i];
+        }
+    }
+}
+
+}  // namespace
+
+GI_API long gi_ssm_state_floats(int inner, int n_state, int n_taps) { return (long)inner * n_state + (long)(n_taps - 1) * inner; }
+GI_API int gi_ssm_max_taps() { return SSM_MAX_TAPS; }
+GI_API int gi_ssm_max_states() { return 256; }
+
+GI_API int gi_ssm_conv(const float* pre, long ld, const float* taps, int n_taps, const float* bias, float* state, long state_stride, int move_tail,
+                       const int* slot, const int* pos, float* x, void* x_low, int low_dtype, int n_rows, int inner, int n_state, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && inner > 0 && n_state > 0 && ld >= inner && n_taps >= 1 && n_taps <= SSM_MAX_TAPS && state_stride >= gi_ssm_state_floats(inner, n_state, n_taps),
+               "ssm_conv: bad sizes (rows %d, channels %d, states %d, taps %d)", n_rows, inner, n_state, n_taps);
+    float* tail = state + (size_t)inner * n_state;
+    dim3 grid(n_rows, (inner + 255) / 256);
+    GI_REQUIRE(grid.y <= 65535, "ssm_conv: too many channels");
+    if (x_low == nullptr || low_dtype == GI_F32) ssm_conv_kernel<float><<<grid, 256, 0, stream>>>(pre, ld, taps, n_taps, bias, tail, state_stride, move_tail, slot, pos, x, (float*)x_low, inner);
+    else if (low_dtype == GI_BF16) ssm_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>(pre, ld, taps, n_taps, bias, tail, state_stride, move_tail, slot, pos, x, (bf16_t*)x_low, inner);
+    else return gi_fail("ssm_conv: unknown dtype %d", low_dtype);
+    GI_CHECK_LAUNCH("ssm_conv");
+    return 0;
+}
+
+GI_API int gi_ssm_tail(const float* pre, long ld, int n_taps, const int* seg_start, const int* seg_len, int n_segs, const int* slot, float* state,
+                       long state_stride, int inner, int n_state, hipStream_t stream) {
+    GI_REQUIRE(n_segs > 0 && inner > 0 && n_state > 0 && ld >= inner && n_taps >= 1 && n_taps <= SSM_MAX_TAPS && state_stride >= gi_ssm_state_floats(inner, n_state, n_taps),
+               "ssm_tail: bad sizes (requests %d, channels %d, taps %d)", n_segs, inner, n_taps);
+    if (n_taps == 1) return 0;
+    dim3 grid(n_segs, min((inner + 255) / 256, 64));
+    ssm_tail_kernel<<<grid, 256, 0, stream>>>(pre, ld, inner, n_taps, seg_start, seg_len, slot, state + (size_t)inner * n_state, state_stride);
+    GI_CHECK_LAUNCH("ssm_tail");
+    return 0;
+}
+
+GI_API int gi_ssm_scan(const float* x, const float* dt_pre, long ld_dt, const float* dt_bias, const float* bc, long ld_bc, int b_off, int c_off, const float* z,
+                       long ld_z, const float* a_log, const float* d_skip, const int* seg_start, const int* seg_len, int n_segs, const int* row_slot,
+                       float* state, long state_stride, void* out, int out_dtype, long ldo, int inner, int n_state, hipStream_t stream) {
+    GI_REQUIRE(n_segs > 0 && inner > 0 && n_state > 0 && n_state <= 256 && ld_dt >= inner && ld_z >= inner && ldo >= inner && b_off >= 0 && c_off >= 0
+               && ld_bc >= b_off + n_state && ld_bc >= c_off + n_state && state_stride >= (long)inner * n_state,
+               "ssm_scan: bad sizes (requests %d, channels %d, states %d)", n_segs, inner, n_state);
+    dim3 grid(n_segs, (inner + 15) / 16);
+    GI_REQUIRE(grid.y <= 65535, "ssm_scan: too many channels");
+#define LAUNCH(NPL, TO)                                                                                                                            \
+    ssm_scan_kernel<NPL, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, seg_len, \
+                                                      row_slot, state, state_stride, (TO*)out, ldo, inner, n_state)
+#define BY_STATES(TO)                                  \
+    do {                                               \
+        if (n_state <= 16) LAUNCH(4, TO);              \
+        else if (n_state <= 32) LAUNCH(8, TO);         \
+        else if (n_state <= 64) LAUNCH(16, TO);        \
+        else if (n_state <= 128) LAUNCH(32, TO);       \
+        else LAUNCH(64, TO);                           \
+    } while (0)
+    if (out_dtype == GI_F32) BY_STATES(float);
+    else if (out_dtype == GI_BF16) BY_STATES(bf16_t);
+    else return gi_fail("ssm_scan: unknown dtype %d", out_dtype);
+#undef BY_STATES
+#undef LAUNCH
+    GI_CHECK_LAUNCH("ssm_scan");
+    return 0;
+}

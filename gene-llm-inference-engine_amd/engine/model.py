@@ -9,7 +9,7 @@ import torch
 
 from ..config import ModelSpec, read_config
 from ..kernels import ops
-from ..parts import LayerCache, StepContext, block_class, linear, model_tensor_needs, norm_class, row_transform_class, weight_bytes
+from ..parts import LayerCache, StepContext, block_class, linear, model_tensor_needs, norm_class, row_transform_class, stream_part_class, weight_bytes
 from ..parts.linear import activation_dtype_for
 from ..parts.norm import HandedRows, norm_to_hand_on
 from ..weights import load_tensors, random_tensors
@@ -48,8 +48,13 @@ class DecoderModel:
         self.after_embedding = [row_transform_class(t)(t, tensors, dtype, device) for t in spec.after_embedding]
         self.after_head = [row_transform_class(t)(t, tensors, dtype, device) for t in spec.after_head]
         self.run_order = spec.run_order
+        # parts that change the residual stream between layers: behind a layer (every time it runs), before a run-order entry
+        self.after_layer = [[stream_part_class(t)(t, tensors, dtype, device) for t in l.after] for l in spec.layers]
+        self.before_entry = [None if e.before is None else stream_part_class(e.before)(e.before, tensors, dtype, device) for e in spec.run_order]
+        stream_parts = [p for parts in self.after_layer for p in parts] + [p for p in self.before_entry if p is not None]
+        self.keeps_token_rows = any(getattr(p, "needs_token_rows", False) for p in stream_parts)
         self.trace = None                        # see set_trace
-        self.graph_safe = all(getattr(p, "graph_safe", False) for p in (*self.layers, self.final_norm, *self.after_embedding, *self.after_head))
+        self.graph_safe = all(getattr(p, "graph_safe", False) for p in (*self.layers, self.final_norm, *self.after_embedding, *self.after_head, *stream_parts))
 
     # ----------------------------------------------------------------------------- what it needs
     def cache_needs(self):
@@ -60,7 +65,8 @@ class DecoderModel:
     def weight_bytes_read_per_step(self) -> int:
         """Bytes of weights one step reads when it uses every matrix once: what every part of the run order holds (a
         layer named twice is read twice), the final norm and the head; the token table is read by row and not counted."""
-        return (sum(weight_bytes(self.layers[e.layer]) for e in self.run_order) + weight_bytes(self.final_norm) + weight_bytes(self.lm_head)
+        return (sum(weight_bytes(self.layers[e.layer]) + weight_bytes(self.after_layer[e.layer]) for e in self.run_order)
+                + weight_bytes([p for p in self.before_entry if p is not None]) + weight_bytes(self.final_norm) + weight_bytes(self.lm_head)
                 + weight_bytes(self.after_embedding) + weight_bytes(self.after_head))
 
     # ------------------------------------------------------------------------------- the pass
@@ -72,11 +78,18 @@ class DecoderModel:
         handed = self._embed(ctx, x)      # the next block's first norm, where whoever wrote x could leave it half applied
         if trace is not None:
             trace("embedding", -1, x)
+        if self.keeps_token_rows:
+            ctx.memo["token_rows"] = x.clone()
         for i, entry in enumerate(self.run_order):
             ctx.trace = None if trace is None else (lambda tag, rows, i=i: trace(tag, i, rows))
-            layer = self.layers[entry.layer]
+            layer, extras = self.layers[entry.layer], self.after_layer[entry.layer]
+            if self.before_entry[i] is not None:          # (it changes x: a norm handed on by whoever wrote x last is void)
+                self.before_entry[i].forward(x, ctx)
+                handed = None
             if getattr(layer, "hands_norm_on", False):
-                if i + 1 < len(self.run_order):
+                if extras or (i + 1 < len(self.run_order) and self.before_entry[i + 1] is not None):
+                    reader = None         # x changes again before anybody reads it
+                elif i + 1 < len(self.run_order):
                     after = self.layers[self.run_order[i + 1].layer]
                     reader = after.first_reader() if getattr(after, "hands_norm_on", False) else None
                 else:                     # the head reads every row of the final norm, or a selection, which is not handed on
@@ -85,6 +98,10 @@ class DecoderModel:
             else:
                 layer.forward(x, ctx, cache.layer_cache(i))
                 handed = None
+            for part in extras:
+                part.forward(x, ctx)
+            if extras and trace is not None:
+                trace("layer_out", i, x)
         ctx.trace = None
         if n_logit_rows == 0:
             return None
@@ -109,7 +126,7 @@ class DecoderModel:
         single rows of decoding requests in bfloat16, a norm of the form g * x * rsqrt(mean square + eps), a reader whose product
         finishes it), the kernel that fetches the rows does the norm's first half too and the `HandedRows` are returned; None otherwise."""
         first = self.layers[self.run_order[0].layer] if self.run_order else None
-        if (first is not None and not self.after_embedding and self.trace is None and self.dtype == torch.bfloat16
+        if (first is not None and not self.after_embedding and self.trace is None and self.dtype == torch.bfloat16 and self.before_entry[0] is None
                 and getattr(first, "hands_norm_on", False) and ctx.max_seg_len == 1):         # (decode steps: the one norm kernel of a step that is all launches)
             norm = norm_to_hand_on(first.first_reader(), ctx.n_rows)
             if norm is not None:

@@ -40,14 +40,14 @@ class _CacheView:
     def __init__(self, manager: CacheManager, needs, reads_from):
         self._layer = []
         for i, (need, src) in enumerate(zip(needs, reads_from)):
-            from ..cache import PagedKvNeed, StateNeed
-            if isinstance(need, PagedKvNeed):
+            from ..cache import paged_need, state_need
+            view = LayerCache()
+            if paged_need(need) is not None:
                 kv, table, _ = manager.kv(i)
-                self._layer.append(LayerCache(kv=kv, table=table, writes=src is None, page_size=manager.page_size))
-            elif isinstance(need, StateNeed):
-                self._layer.append(LayerCache(state=manager.state(i)))
-            else:
-                self._layer.append(LayerCache())
+                view = LayerCache(kv=kv, table=table, writes=src is None, page_size=manager.page_size)
+            if state_need(need) is not None:
+                view.state = manager.state(i)
+            self._layer.append(view)
 
     def layer_cache(self, entry: int) -> LayerCache:
         return self._layer[entry]

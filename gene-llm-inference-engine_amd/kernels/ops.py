@@ -40,7 +40,18 @@ _SIGNATURES = {
     "gi_rmsnorm_add_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_long, c_long, c_long, c_void_p],
     "gi_norm_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int,
                            c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p],
+                           c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_void_p],
+    "gi_concat_rows": [c_void_p, c_long, c_int, c_void_p, c_long, c_int, c_void_p, c_int, c_long, c_int, c_void_p],
+    "gi_add_weighted": [c_void_p, c_long, c_void_p, c_long, c_float, c_void_p, c_long, c_float, c_int, c_int, c_void_p],
+    "gi_add_vector": [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
+    "gi_gate_token_columns": [c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_void_p],
+    "gi_ssm_conv": [c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_ssm_tail": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p],
+    "gi_ssm_scan": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                    c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p],
+    "gi_route_top": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_experts_down": [c_void_p, c_int, c_long, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_xielu": [c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p, c_void_p],
     "gi_delta_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
                          c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
@@ -494,14 +505,17 @@ def rmsnorm_add_norm(y, weight, eps, x, next_weight, next_eps, out):
 
 
 def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, positions, slots, table, q_out, cache, page_size, n_heads, n_kv, hd, vd,
-                    biases=None, blend=None, keep=None):
+                    biases=None, blend=None, keep=None, neighbours=False, unit_rms=False, norm_last=False):
     """The general form of `rope_store`: every query and key head is first RMS-normed with q_norm / k_norm [hd] (None: not), then
     the pairs (i, i + rotary_dim/2) of its first rotary_dim channels are turned (cos, sin float32 [n, rotary_dim/2]; None: not);
     queries go to q_out, keys and the values (vd channels a head) into the cache's pages.  k None: the pages are another layer's.
     biases = (q_bias, k_bias, v_bias): float32 vectors added to the products first (each may be None).  blend = (other, weight):
     the values that go into the pages are (1 - weight) v + weight other, other float32 [n, kv_heads*vd] (another layer's values of
     the same rows), weight one float32 number on the device.  keep: float32 [n, kv_heads*vd], gets this layer's values (with
-    their bias, before any blending)."""
+    their bias, before any blending).  neighbours: the pairs turned are (2i, 2i + 1).  unit_rms: every query and key head is divided
+    by its root mean square (eps inside the root), without weights.  norm_last: the heads' norm comes behind the rotation."""
+    if unit_rms and (q_norm is not None or k_norm is not None):
+        raise KernelError("norm_rope_store: heads divided by their root mean square have no norm weights")
     _dev(q, k, v, q_norm, k_norm, cos, sin, positions, slots, table, q_out, cache)
     q_bias, k_bias, v_bias = biases if biases is not None else (None, None, None)
     other, weight = blend if blend is not None else (None, None)
@@ -544,7 +558,7 @@ def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, position
           slots.data_ptr(), _ptr(table) if k is not None else None, table.stride(0) if k is not None else 0, q_out.data_ptr(),
           _code(q_out, "norm_rope_store: q_out"), _ptr(cache) if k is not None else None, cache_code, cache.stride(0) if k is not None else 0,
           int(page_size), n, n_heads, n_kv, hd, vd, _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), _ptr(other), other.stride(0) if other is not None else 0,
-          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, _stream())
+          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, (1 if neighbours else 0) | (2 if unit_rms else 0) | (4 if norm_last else 0), _stream())
 
 
 def xielu(x, out, params):
@@ -1387,3 +1401,187 @@ def latent_attention_bf16(q, cache, out, ctx, table, n_heads, kd, vd, page_size,
     _call("gi_latent_attention_bf16", q.data_ptr(), cache.data_ptr(), out.data_ptr(), _ptr(part), n_part, _ptr(rows), ctx.row_pos.data_ptr(), ctx.row_slot.data_ptr(),
           table.data_ptr(), table.stride(0), cache.stride(0), int(page_size), n_single, n_heads, kd, vd, int(window or 0), float(scale), n_splits, _stream())
     return out
+
+
+# --------------------------------------------------------------------------- rows side by side, weighted sums, a vector on every row
+def _f32_rows(t, what, n=None, width=None):
+    if t is None:
+        return
+    if not (t.dtype == torch.float32 and t.dim() == 2 and t.stride(1) == 1 and (n is None or t.shape[0] == n) and (width is None or t.shape[1] == width)):
+        raise KernelError(f"{what} must be float32 [{n if n is not None else 'n'}, {width if width is not None else 'width'}] with unit inner stride")
+
+
+def concat_rows(a, b, out):
+    """out[t] = [a[t]; b[t]] (b None: a alone), float32 rows stored as `out`'s dtype."""
+    _dev(a, b, out)
+    n, wa = a.shape
+    wb = 0 if b is None else b.shape[1]
+    _f32_rows(a, "concat_rows: a")
+    _f32_rows(b, "concat_rows: b", n)
+    if not (out.shape == (n, wa + wb) and out.stride(1) == 1):
+        raise KernelError("concat_rows: out must be [n, columns of both] with unit inner stride")
+    _call("gi_concat_rows", a.data_ptr(), a.stride(0), wa, _ptr(b), b.stride(0) if b is not None else 0, wb, out.data_ptr(), _code(out, "concat_rows: out"),
+          out.stride(0), n, _stream())
+    return out
+
+
+def add_weighted(x, a, scale_a, b=None, scale_b=0.0):
+    """x += scale_a * a + scale_b * b (float32 rows; b may be None)."""
+    _dev(x, a, b)
+    n, dim = x.shape
+    _f32_rows(x, "add_weighted: x")
+    _f32_rows(a, "add_weighted: a", n, dim)
+    _f32_rows(b, "add_weighted: b", n, dim)
+    _call("gi_add_weighted", x.data_ptr(), x.stride(0), a.data_ptr(), a.stride(0), float(scale_a), _ptr(b), b.stride(0) if b is not None else 0, float(scale_b), n, dim, _stream())
+    return x
+
+
+def add_vector(x, v):
+    """x[t] += v for every row."""
+    _dev(x, v)
+    n, dim = x.shape
+    _f32_rows(x, "add_vector: x")
+    if not (v.shape == (dim,) and v.is_contiguous()):
+        raise KernelError("add_vector: the vector must be [dim], contiguous")
+    _call("gi_add_vector", x.data_ptr(), x.stride(0), v.data_ptr(), _code(v, "add_vector: v"), n, dim, _stream())
+    return x
+
+
+def gate_token_columns(u, table, first, tokens, out, activation="gelu_tanh"):
+    """out[t, c] = act(u[t, c]) * table[tokens[t], first + c]."""
+    _dev(u, table, tokens, out)
+    n, dim = u.shape
+    _f32_rows(u, "gate_token_columns: u")
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"gate_token_columns: unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
+    if not (table.dim() == 2 and table.stride(1) == 1 and 0 <= first and first + dim <= table.shape[1] and out.shape == (n, dim) and out.stride(1) == 1):
+        raise KernelError("gate_token_columns: the table must hold the columns asked for, out must be [n, dim]")
+    _i32(tokens, "gate_token_columns: tokens", n)
+    _call("gi_gate_token_columns", u.data_ptr(), u.stride(0), table.data_ptr(), _code(table, "gate_token_columns: table"), table.stride(0), int(first), tokens.data_ptr(),
+          out.data_ptr(), _code(out, "gate_token_columns: out"), out.stride(0), n, dim, ACTIVATIONS[activation], _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------------------ the selective scan
+SSM_MAX_TAPS, SSM_MAX_STATES = 8, 256
+
+
+def ssm_state_floats(inner, n_state, n_taps) -> int:
+    """32-bit numbers of one request's state: S [inner][n_state], then the convolution's last n_taps - 1 inputs [n_taps - 1][inner]."""
+    return inner * n_state + (n_taps - 1) * inner
+
+
+def _ssm_state(state, inner, n_state, n_taps, what):
+    if not (state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] >= ssm_state_floats(inner, n_state, n_taps)):
+        raise KernelError(f"{what}: the state must be float32 [slots, {ssm_state_floats(inner, n_state, n_taps)}]")
+
+
+def ssm_conv(pre, taps, bias, ctx_slots, ctx_positions, state, x, x_low, n_state, move_tail=False):
+    """x = SiLU(convolution of `pre` [n, inner] over each request's rows + bias), float32, and the same once more as `x_low`'s dtype
+    (None: not).  taps float32 [inner, n_taps]; rows before a step come from the request's state.  move_tail: a step of single rows,
+    whose kernel also moves every request's tail on."""
+    _dev(pre, taps, bias, ctx_slots, ctx_positions, state, x, x_low)
+    n, inner = x.shape
+    n_taps = taps.shape[1]
+    _f32_rows(pre, "ssm_conv: the projection", n, inner)
+    if not (x.dtype == torch.float32 and x.is_contiguous() and (x_low is None or (x_low.shape == (n, inner) and x_low.is_contiguous()))):
+        raise KernelError("ssm_conv: x (and its copy) must be [n, inner], contiguous")
+    if not (taps.dtype == torch.float32 and taps.shape == (inner, n_taps) and taps.is_contiguous() and bias.dtype == torch.float32 and bias.shape == (inner,) and bias.is_contiguous()):
+        raise KernelError("ssm_conv: taps must be float32 [inner, taps] and the bias float32 [inner]")
+    if not 1 <= n_taps <= SSM_MAX_TAPS:
+        raise KernelError(f"ssm_conv: {n_taps} taps are outside what the kernel takes (1 to {SSM_MAX_TAPS})")
+    _ssm_state(state, inner, n_state, n_taps, "ssm_conv")
+    _i32(ctx_slots, "ssm_conv: slots", n)
+    _i32(ctx_positions, "ssm_conv: positions", n)
+    _call("gi_ssm_conv", pre.data_ptr(), pre.stride(0), taps.data_ptr(), n_taps, bias.data_ptr(), state.data_ptr(), state.stride(0), 1 if move_tail else 0,
+          ctx_slots.data_ptr(), ctx_positions.data_ptr(), x.data_ptr(), _ptr(x_low), _code(x_low, "ssm_conv: copy") if x_low is not None else F32, n, inner, n_state, _stream())
+
+
+def ssm_tail(pre, n_taps, seg_start, seg_len, row_slot, state, inner, n_state):
+    """Every request's last n_taps - 1 convolution inputs, moved on behind `ssm_conv`."""
+    _dev(pre, seg_start, seg_len, row_slot, state)
+    _f32_rows(pre, "ssm_tail: the projection", None, inner)
+    _ssm_state(state, inner, n_state, n_taps, "ssm_tail")
+    _call("gi_ssm_tail", pre.data_ptr(), pre.stride(0), n_taps, seg_start.data_ptr(), seg_len.data_ptr(), seg_start.numel(), row_slot.data_ptr(), state.data_ptr(),
+          state.stride(0), inner, n_state, _stream())
+
+
+def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out, n_state):
+    """The recurrence over every request's rows, from its state slot and back into it; out [n, inner] = (read-out + D x) * SiLU(z).
+    x float32 [n, inner] contiguous; dt_pre, z float32 [n, inner] (any row stride); low float32 [n, >= offsets + n_state] holds B and
+    C of every row at the two offsets; dt_bias, d_skip float32 [inner]; a_log float32 [inner, n_state]."""
+    _dev(x, dt_pre, dt_bias, low, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out)
+    n, inner = x.shape
+    _f32_rows(dt_pre, "ssm_scan: the step sizes", n, inner)
+    _f32_rows(z, "ssm_scan: the gate", n, inner)
+    _f32_rows(low, "ssm_scan: B and C", n)
+    if not (x.dtype == torch.float32 and x.is_contiguous() and out.shape == (n, inner) and out.stride(1) == 1):
+        raise KernelError("ssm_scan: x must be float32 [n, inner], contiguous, and out [n, inner]")
+    if not 1 <= n_state <= SSM_MAX_STATES or max(b_off, c_off) + n_state > low.shape[1] or min(b_off, c_off) < 0:
+        raise KernelError(f"ssm_scan: {n_state} states at columns {b_off} and {c_off} of {low.shape[1]} are outside what the kernel takes")
+    for v, shape, name in ((dt_bias, (inner,), "dt_bias"), (d_skip, (inner,), "D"), (a_log, (inner, n_state), "A_log")):
+        if not (v.dtype == torch.float32 and v.shape == shape and v.is_contiguous()):
+            raise KernelError(f"ssm_scan: {name} must be float32 {list(shape)}")
+    _ssm_state(state, inner, n_state, 1, "ssm_scan")
+    _i32(row_slot, "ssm_scan: slots", n)
+    _call("gi_ssm_scan", x.data_ptr(), dt_pre.data_ptr(), dt_pre.stride(0), dt_bias.data_ptr(), low.data_ptr(), low.stride(0), int(b_off), int(c_off), z.data_ptr(),
+          z.stride(0), a_log.data_ptr(), d_skip.data_ptr(), seg_start.data_ptr(), seg_len.data_ptr(), seg_start.numel(), row_slot.data_ptr(), state.data_ptr(),
+          state.stride(0), out.data_ptr(), _code(out, "ssm_scan: out"), out.stride(0), inner, n_state, _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------------------------ routed experts
+ROUTER_SCORES = {"sigmoid": 0, "softmax": 1}
+ROUTER_MAX_EXPERTS, ROUTER_MAX_TOP = 1024, 64
+
+
+def route_top(logits, top, ids, weights, score="sigmoid", renormalize=False):
+    """ids int32 [n, top], weights float32 [n, top]: per row the `top` experts with the largest scores (the lower index wins a tie)
+    and their scores, divided by their sum if `renormalize`."""
+    _dev(logits, ids, weights)
+    n, n_experts = logits.shape
+    _f32_rows(logits, "route_top: logits")
+    if score not in ROUTER_SCORES:
+        raise KernelError(f"route_top: unknown score {score!r}; known: {', '.join(ROUTER_SCORES)}")
+    if not (1 <= top <= min(n_experts, ROUTER_MAX_TOP) and n_experts <= ROUTER_MAX_EXPERTS):
+        raise KernelError(f"route_top: top {top} of {n_experts} experts is outside what the kernel takes")
+    if not (ids.dtype == torch.int32 and ids.shape == (n, top) and ids.is_contiguous() and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()):
+        raise KernelError("route_top: ids must be int32 [n, top] and weights float32 [n, top], contiguous")
+    _call("gi_route_top", logits.data_ptr(), logits.stride(0), n, n_experts, top, ROUTER_SCORES[score], 1 if renormalize else 0, ids.data_ptr(), weights.data_ptr(), _stream())
+
+
+def _expert_stack(w, rows, cols, what):
+    if not (w.dim() == 3 and w.shape[1:] == (rows, cols) and w.is_contiguous()):
+        raise KernelError(f"{what} must be [experts, {rows}, {cols}], contiguous")
+
+
+def experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=True, activation="silu"):
+    """mid[(row, choice)] = act(W_gate[e] a) * (W_up[e] a), a = the row of h (times the choice's weight if `weigh_input`, stored as
+    h's dtype), e = ids[row, choice]; one wave per output, for the few rows of decoding steps."""
+    _dev(h, w_gate, w_up, ids, weights, mid)
+    n, width = h.shape
+    top, ff = ids.shape[1], w_gate.shape[1]
+    _expert_stack(w_gate, ff, width, "experts_gate_up: the gates")
+    _expert_stack(w_up, ff, width, "experts_gate_up: the up products")
+    if not (h.stride(1) == 1 and mid.shape == (n * top, ff) and mid.stride(1) == 1 and w_gate.dtype == w_up.dtype and ids.dtype == torch.int32 and ids.is_contiguous()
+            and ids.shape == (n, top) and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()):
+        raise KernelError("experts_gate_up: h [n, width], mid [n * top, ff], ids int32 and weights float32 [n, top] are needed")
+    _call("gi_experts_gate_up", h.data_ptr(), _code(h, "experts_gate_up: h"), h.stride(0), w_gate.data_ptr(), w_up.data_ptr(), _code(w_gate, "experts_gate_up: weights"),
+          ids.data_ptr(), weights.data_ptr(), 1 if weigh_input else 0, mid.data_ptr(), _code(mid, "experts_gate_up: mid"), mid.stride(0), n, top, width, ff,
+          ACTIVATIONS[activation], _stream())
+    return mid
+
+
+def experts_down(mid, w_down, ids, weights, x, accumulate=True, weigh_output=False):
+    """x[row] (+)= sum over the row's choices of W_down[e] mid[(row, choice)] (times the choice's weight if `weigh_output`)."""
+    _dev(mid, w_down, ids, weights, x)
+    n, width = x.shape
+    top, ff = ids.shape[1], w_down.shape[2]
+    _expert_stack(w_down, width, ff, "experts_down: the down products")
+    _f32_rows(x, "experts_down: x")
+    if not (mid.shape == (n * top, ff) and mid.stride(1) == 1 and ids.dtype == torch.int32 and ids.shape == (n, top) and ids.is_contiguous()
+            and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()):
+        raise KernelError("experts_down: mid [n * top, ff], ids int32 and weights float32 [n, top] are needed")
+    _call("gi_experts_down", mid.data_ptr(), _code(mid, "experts_down: mid"), mid.stride(0), w_down.data_ptr(), _code(w_down, "experts_down: weights"), ids.data_ptr(),
+          weights.data_ptr(), 1 if weigh_output else 0, x.data_ptr(), x.stride(0), 1 if accumulate else 0, n, top, width, ff, _stream())
+    return x

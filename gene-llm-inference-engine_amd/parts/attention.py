@@ -120,8 +120,14 @@ class Attention(Mixer):
             self.value_blend = None if s.value_blend is None else tensors[s.value_blend].float().reshape(1).contiguous()
             if s.value_blend is not None and s.value_family is None:
                 raise ValueError("attention: a blend of values needs the family whose first layer's values are blended in")
-            if self.position is not None and not (hasattr(self.position, "partial_tables") or type(self.position).half_split_tables is not PositionEncoding.half_split_tables):
-                if self.q_norm is not None or self.k_norm is not None:
+            self.unit_rms = bool(getattr(s, "qk_unit_rms", False))
+            if self.unit_rms and (self.q_norm is not None or self.k_norm is not None):
+                raise ValueError("attention: heads divided by their root mean square have no norm weights")
+            if self.position is not None and hasattr(self.position, "pair_tables") and self.position.rotary_dim > s.head_dim:
+                raise ValueError("attention: more channels to turn than a head has")
+            if self.position is not None and not (hasattr(self.position, "partial_tables") or hasattr(self.position, "pair_tables")
+                                                  or type(self.position).half_split_tables is not PositionEncoding.half_split_tables):
+                if self.q_norm is not None or self.k_norm is not None or self.unit_rms:
                     raise ValueError("attention: norms on query and key heads come before the rotation, which needs a position encoding that hands over its cosines and sines")
         else:
             self.w_qkv = torch.cat([tensors[s.q_proj], tensors[s.k_proj], tensors[s.v_proj]], dim=0).contiguous()
@@ -134,7 +140,7 @@ class Attention(Mixer):
     def _is_general(s) -> bool:
         return (s.k_proj is None or any(v is not None for v in (s.value_dim, s.scale, s.chunk, s.sinks, s.q_norm, s.k_norm, s.head_gate, s.q_bias,
                                                                  s.k_bias, s.v_bias, s.value_family, s.value_blend))
-                or getattr(s.position, "kind", None) == "rotary_partial")
+                or getattr(s, "qk_unit_rms", False) or getattr(s.position, "kind", None) in ("rotary_partial", "rotary_interleaved"))
 
     @classmethod
     def tensor_needs(cls, spec):
@@ -188,7 +194,8 @@ class Attention(Mixer):
         if s.k_proj is not None and cache.writes:
             k, v = proj[:, self.a_dim:self.a_dim + self.kv_dim], proj[:, self.a_dim + self.kv_dim:self.a_dim + self.kv_dim + s.n_kv_heads * vd]
         gate = proj[:, self.gate_at:self.gate_at + s.n_heads] if s.head_gate is not None else None
-        tables = rotation_tables(self.position, ctx)
+        neighbours = self.position is not None and hasattr(self.position, "pair_tables")          # pairs (2i, 2i + 1) of a head's first channels
+        tables = (*self.position.pair_tables(ctx), self.position.rotary_dim) if neighbours else rotation_tables(self.position, ctx)
         if self.position is not None and tables is None:          # an encoding with kernels of its own turns q and k in place
             self.position.apply(q, k, ctx, s.n_heads, s.n_kv_heads, s.head_dim)
         cos, sin, turned = tables if tables is not None else (None, None, 0)
@@ -205,7 +212,8 @@ class Attention(Mixer):
         biases = self.biases if k is not None else (self.biases[0], None, None)
         ops.norm_rope_store(q, k, v, self.q_norm, self.k_norm if k is not None else None, s.qk_norm_eps, cos, sin, turned, ctx.row_pos, ctx.row_slot,
                             cache.table, q_ready, cache.kv, cache.page_size, s.n_heads, s.n_kv_heads, s.head_dim, vd,
-                            biases=biases if any(b is not None for b in biases) else None, blend=blend, keep=keep)
+                            biases=biases if any(b is not None for b in biases) else None, blend=blend, keep=keep, neighbours=neighbours,
+                            unit_rms=self.unit_rms, norm_last=self.unit_rms)
         att = torch.empty((T, s.n_heads * vd), dtype=cache.kv.dtype, device=ctx.device)
         return ops.attention_general(q_ready, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, page_size=cache.page_size,
                                      value_dim=vd, window=s.window, chunk=s.chunk, scale=s.scale, sinks=self.sinks, gate=gate)

@@ -17,6 +17,10 @@ Kinds of parts and what each must provide:
 * feed-forward:      `tensor_needs(spec)`, `forward(h, residual, ctx)`
 * block:             `forward(x, ctx, cache)` wiring norms, mixer and feed-forward around the
                      32-bit residual stream `x`
+* stream part:       `tensor_needs(spec)`, `forward(x, ctx)` changes the residual stream in place, behind a layer
+                     (`LayerSpec.after`) or before a run-order entry (`RunEntry.before`); one that says
+                     `needs_token_rows` finds the rows of the token table, as the first layer got them, in
+                     `ctx.memo["token_rows"]`
 
 Mixers and feed-forwards add their result onto `residual` (float32 [T, hidden]) in place.
 """
@@ -105,7 +109,7 @@ class Mixer(Part):
 
     @classmethod
     def cache_need(cls, spec):
-        """A `PagedKvNeed`, a `StateNeed` or None."""
+        """A `PagedKvNeed`, a `StateNeed`, a `JointNeed` of both, or None."""
         return None
 
     def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
@@ -162,6 +166,16 @@ class PositionEncoding(Part):
         raise NotImplementedError(f"{type(self).__name__} gives neither half-split tables nor an apply step")
 
 
+class StreamPart(Part):
+    """Something that changes the residual stream x (float32 [T, hidden]) in place between layers: a second input from the
+    tokens, a product that mixes the stream with the token rows again.  It reads what it needs of the step from `ctx` (the
+    tokens on the device; `ctx.memo["token_rows"]`, float32 [T, hidden], if it says `needs_token_rows`)."""
+    needs_token_rows = False
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> None:
+        raise NotImplementedError
+
+
 class RowTransform(Part):
     """An elementwise change of float32 rows in place: what a model may ask for between the token table and the
     first layer, and on the logits."""
@@ -202,7 +216,7 @@ def weight_bytes(obj) -> int:
     return sum(by_address.values())
 
 
-_REGISTRIES: Dict[str, Dict[str, type]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "row_transform": {}}
+_REGISTRIES: Dict[str, Dict[str, type]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "row_transform": {}, "stream_part": {}}
 
 
 def _register(family: str, kind: str, cls: type) -> None:
@@ -225,6 +239,7 @@ def register_norm(kind, cls): _register("norm", kind, cls)
 def register_position_encoding(kind, cls): _register("position", kind, cls)
 def register_block(kind, cls): _register("block", kind, cls)
 def register_row_transform(kind, cls): _register("row_transform", kind, cls)
+def register_stream_part(kind, cls): _register("stream_part", kind, cls)
 
 
 def mixer_class(spec): return _lookup("mixer", spec.kind)
@@ -233,3 +248,4 @@ def norm_class(spec): return _lookup("norm", spec.kind)
 def position_class(spec): return _lookup("position", spec.kind)
 def block_class(kind: str): return _lookup("block", kind)
 def row_transform_class(spec): return _lookup("row_transform", spec.kind)
+def stream_part_class(spec): return _lookup("stream_part", spec.kind)

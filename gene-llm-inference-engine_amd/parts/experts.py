@@ -1,0 +1,77 @@
+"""A mixture of gated feed-forwards behind a router (`config.spec.RoutedExpertsSpec` states the rules; kernels: `csrc/experts.hip`).
+
+The router's logits are a 32-bit product of the normed rows (as the compute dtype stores them) with the router's matrix; one
+kernel turns them into every row's choice of experts and their weights.  The experts' matrices lie in three stacks
+[experts, ...], and every (row, choice) walks its own expert's: nothing of a step's shape depends on the router's choices, so a
+captured pass may contain the part.  A shared feed-forward, if the spec names one, is a part of its own kind and adds onto the
+same rows."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from ..weights.loader import TensorNeed
+from .base import FeedForward, feed_forward_class, register_feed_forward
+from .linear import activation_dtype_for, linear
+from .norm import NormedRows
+
+
+class RoutedExperts(FeedForward):
+    graph_safe = True
+    can_overwrite = True
+
+    def __init__(self, spec, tensors, dtype, device):
+        super().__init__(spec, tensors, dtype, device)
+        s = spec
+        if s.score not in ops.ROUTER_SCORES:
+            raise ValueError(f"routed experts: unknown score {s.score!r}; known: {', '.join(ops.ROUTER_SCORES)}")
+        if s.weigh not in ("input", "output"):
+            raise ValueError(f"routed experts: the weights weigh an expert's 'input' or its 'output', not {s.weigh!r}")
+        if s.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"routed experts: unknown activation {s.activation!r}; known: {', '.join(ops.ACTIVATIONS)}")
+        if s.n_experts > ops.ROUTER_MAX_EXPERTS or s.top > ops.ROUTER_MAX_TOP:
+            raise ValueError(f"routed experts: at most {ops.ROUTER_MAX_EXPERTS} experts and {ops.ROUTER_MAX_TOP} a row")
+        self.router = tensors[s.router]
+        self.w_gate = torch.stack([tensors[n] for n in s.gate_projs]).contiguous()
+        self.w_up = torch.stack([tensors[n] for n in s.up_projs]).contiguous()
+        self.w_down = torch.stack([tensors[n] for n in s.down_projs]).contiguous()
+        self.in_dtype = activation_dtype_for(self.w_gate, dtype)
+        self.mid_dtype = activation_dtype_for(self.w_down, dtype)
+        self.shared = None if s.shared is None else feed_forward_class(s.shared)(s.shared, tensors, dtype, device)
+        if self.shared is not None and getattr(self.shared, "in_dtype", self.in_dtype) != self.in_dtype:
+            raise ValueError("routed experts: the shared feed-forward must read rows stored as the experts read them")
+        self.graph_safe = self.shared is None or bool(getattr(self.shared, "graph_safe", False))
+
+    @classmethod
+    def tensor_needs(cls, spec):
+        s, d, i = spec, spec.hidden_size, spec.intermediate_size
+        needs = [TensorNeed(s.router, (s.n_experts, d))]
+        for g, u, w in zip(s.gate_projs, s.up_projs, s.down_projs):
+            needs += [TensorNeed(g, (i, d)), TensorNeed(u, (i, d)), TensorNeed(w, (d, i))]
+        if s.shared is not None:
+            needs += feed_forward_class(s.shared).tensor_needs(s.shared)
+        return needs
+
+    def weights_read_per_step(self):
+        """What a step of few rows reads: the router, `top` experts a row at most (here: of one row), the shared feed-forward."""
+        s = self.spec
+        share = [w[:min(s.top, s.n_experts)] for w in (self.w_gate, self.w_up, self.w_down)]
+        return [self.router, *share] + ([self.shared] if self.shared is not None else [])
+
+    def forward(self, h, residual, ctx, then=None, overwrite=False):
+        s, T, dev = self.spec, ctx.n_rows, ctx.device
+        rows = h.materialize() if isinstance(h, NormedRows) else h
+        logits = torch.empty((T, s.n_experts), dtype=torch.float32, device=dev)
+        ops.gemm_exact(rows, self.router, logits)
+        ids = torch.empty((T, s.top), dtype=torch.int32, device=dev)
+        weights = torch.empty((T, s.top), dtype=torch.float32, device=dev)
+        ops.route_top(logits, s.top, ids, weights, s.score, s.renormalize)
+        mid = torch.empty((T * s.top, s.intermediate_size), dtype=self.mid_dtype, device=dev)
+        ops.experts_gate_up(rows, self.w_gate, self.w_up, ids, weights, mid, weigh_input=s.weigh == "input", activation=s.activation)
+        ops.experts_down(mid, self.w_down, ids, weights, residual, accumulate=not overwrite, weigh_output=s.weigh == "output")
+        if self.shared is not None:
+            self.shared.forward(rows, residual, ctx)
+        return None
+
+
+register_feed_forward("routed_experts", RoutedExperts)
