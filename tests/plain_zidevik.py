@@ -192,3 +192,16 @@ def run_model(config, w, tokens, store=same, streams=None):
     logits = store(rms_norm(x, w["final.norm"], eps)) @ w["head"].T
     cap = config.get("logit_softcap")
     return softcap(logits, cap) if cap else logits
+
+
+def forward(config, stored, tokens, dtype=torch.float64, store=same, streams=None):
+    """Logits [T, vocab] from tensors as a file stores them, computed in `dtype`."""
+    w = {k: v.to(dtype) if v.is_floating_point() else v for k, v in stored.items()}
+    return run_model(config, w, tokens, store=store, streams=streams)
+
+
+def greedy(config, stored, prompt, n_new):
+    tokens = list(prompt)
+    for _ in range(n_new):
+        tokens.append(int(forward(config, stored, tokens)[-1].argmax()))
+    return tokens[len(prompt):]
