@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--config FILE] [--prefill-tokens T] [--layers L] [--no-points]
     python bench.py --fekorax [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]     (another record: see `fekorax_beside_llama`)
     python bench.py --rigalorn [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]    (another record: see `rigalorn_beside_fekorax`)
+    python bench.py --zidevik [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]     (another record: see `zidevik_beside_rigalorn`)
 
 A step is one decode step of the whole batch (default batch 8, each request on a 2,048-token
 prompt in a 4,096-token context), through the scheduler with its defaults.  After W warm-up steps,
@@ -175,6 +176,47 @@ def rigalorn_beside_fekorax(args) -> int:
     return 0
 
 
+def zidevik_beside_rigalorn(args) -> int:
+    """The Zidevik design at layer shapes of real models beside the Rigalorn design (the nearest the engine has: parallel layers,
+    attention and recurrences with short convolutions) and the Llama decoder at the same shapes, random weights; measured as
+    `fekorax_beside_llama` measures.  Every Zidevik layer here has the Llama layer's attention heads (pairs of neighbours turned in
+    half of each head, unit heads) beside a selective scan of twice the width with 16 states a channel, step sizes of rank width/16
+    and 4 taps; the feed-forwards take turns: the Llama layer's dense one, then 8 experts of a quarter of its inner size, of which 2
+    serve a token, with a shared expert of half of it (as many weights at work a token as the dense one).  Every layer reads 256
+    columns of the tokens' second table.  Layers 0 and 1 are walked twice, so a model of L layers here runs L + 2.  The Rigalorn
+    model is `rigalorn_beside_fekorax`'s.  One JSON line."""
+    import torch
+    T, batch, L, steps = args.prefill_tokens, args.batch, args.layers or 8, args.steps
+    gen = torch.Generator().manual_seed(1)
+    record = {"metric": "Zidevik beside Rigalorn and Llama at equal layer shapes: prefill tok/s, decode ms a step, ms by kernel", "dtype": args.dtype, "layers": L,
+              "prefill_tokens": T, "decode_batch": batch, "data": "synthetic: random weights by formula, uniform random token ids", "sizes": {}}
+    for size in args.sizes.split(","):
+        D, H, G, hd, ff, vocab = FEKORAX_SIZES[size]
+        mlp = dict(kind="dense", ff=ff)
+        llama = dict(architectures=["LlamaForCausalLM"], hidden_size=D, intermediate_size=ff, num_hidden_layers=L, num_attention_heads=H,
+                     num_key_value_heads=G, head_dim=hd, vocab_size=vocab, max_position_embeddings=T + 1024, rope_theta=500000.0, rms_norm_eps=1e-5,
+                     tie_word_embeddings=True)
+        delta = dict(type="delta", mlp=mlp, mixer=dict(heads=max(1, H // 4), kv_heads=max(1, H // 8), dim=hd, vdim=2 * hd, conv=4))
+        latent = dict(type="latent_attention", mlp=mlp, mixer=dict(heads=H, dim=hd, rot_dim=hd // 2, vdim=hd, q_rank=12 * hd, kv_rank=4 * hd, scale=(1.5 * hd) ** -0.5,
+                                                                    rot=dict(dims=hd // 2, base=500000.0), mask=dict(size=1024)))
+        blended = dict(type="attention", mlp=mlp, mixer=dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, v_mix=True, mask=dict(size=1024), rot=dict(
+            dims=hd // 2, base=10000.0, scaling=dict(factor=4.0, original=4096, fast=16.0, slow=2.0))))
+        rigalorn = dict(architecture="Rigalorn", vocab=vocab, width=D, embedding=dict(scale=D ** 0.5), norm=dict(eps=1e-5), max_positions=T + 1024,
+                        layers=([delta, latent, blended, delta] * ((L + 3) // 4))[:L])
+        mixer = dict(left=dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, rot=dict(dims=hd // 2, base=500000.0)), left_scale=1.0,
+                     right=dict(inner=2 * D, state=16, dt_rank=D // 16, conv=4), right_scale=1.0)
+        moe = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=ff // 4), shared=dict(ff=ff // 2))
+        zidevik = dict(architecture="Zidevik", vocab=vocab, width=D, norm=dict(eps=1e-5), max_positions=T + 1024, logit_softcap=30.0, token_side=dict(dim=256),
+                       loop=dict(start=0, stop=min(2, L), times=2), layers=[dict(type="parallel", mixer=mixer, mlp=mlp if i % 2 == 0 else moe) for i in range(L)])
+        record["sizes"][size] = {}
+        for name, cfg in (("llama", llama), ("rigalorn", rigalorn), ("zidevik", zidevik)):
+            if args.only and name not in args.only.split(","):
+                continue
+            record["sizes"][size][name] = _measure_design(cfg, args, T, batch, steps, vocab, gen)
+    print(json.dumps(record))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -188,8 +230,9 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=PROMPT, help="length of the timed prompt")
     ap.add_argument("--fekorax", action="store_true", help="another measurement: the Fekorax design beside Llama at equal layer shapes (see fekorax_beside_llama)")
     ap.add_argument("--rigalorn", action="store_true", help="another measurement: the Rigalorn design beside Fekorax and Llama at equal layer shapes (see rigalorn_beside_fekorax)")
-    ap.add_argument("--only", default="", help="with --rigalorn: the designs to measure, of llama, fekorax, rigalorn (default: all)")
-    ap.add_argument("--sizes", default="1b,8b", help="with --fekorax or --rigalorn: layer shapes, of " + ", ".join(FEKORAX_SIZES))
+    ap.add_argument("--zidevik", action="store_true", help="another measurement: the Zidevik design beside Rigalorn and Llama at equal layer shapes (see zidevik_beside_rigalorn)")
+    ap.add_argument("--only", default="", help="with --rigalorn or --zidevik: the designs to measure, of llama, fekorax, rigalorn, zidevik (default: all)")
+    ap.add_argument("--sizes", default="1b,8b", help="with --fekorax, --rigalorn or --zidevik: layer shapes, of " + ", ".join(FEKORAX_SIZES))
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
@@ -199,6 +242,8 @@ def main() -> int:
         return fekorax_beside_llama(args)
     if args.rigalorn:
         return rigalorn_beside_fekorax(args)
+    if args.zidevik:
+        return zidevik_beside_rigalorn(args)
 
     import torch
     from geneinfer_amd.config import LlamaConfig

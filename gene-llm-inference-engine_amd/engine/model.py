@@ -100,7 +100,7 @@ class DecoderModel:
                 handed = None
             for part in extras:
                 part.forward(x, ctx)
-            if extras and trace is not None:
+            if trace is not None:
                 trace("layer_out", i, x)
         ctx.trace = None
         if n_logit_rows == 0:
@@ -142,7 +142,7 @@ class DecoderModel:
     def set_trace(self, trace) -> None:
         """Debugging, as the reference's Model::set_trace (src/model/model.h): `trace(tag, run-order entry or -1, rows)` is
         called with the step's residual stream after the embedding ("embedding"), after each half of every block
-        ("attn_out", "ffn_out") and with the normed rows that the logits are taken from ("final_norm").  While a trace is
+        ("attn_out", "ffn_out"), after everything that belongs to a run-order entry ("layer_out") and with the normed rows that the logits are taken from ("final_norm").  While a trace is
         set no step is replayed from a captured graph."""
         self.trace = trace
 

@@ -1585,3 +1585,17 @@ def experts_down(mid, w_down, ids, weights, x, accumulate=True, weigh_output=Fal
     _call("gi_experts_down", mid.data_ptr(), _code(mid, "experts_down: mid"), mid.stride(0), w_down.data_ptr(), _code(w_down, "experts_down: weights"), ids.data_ptr(),
           weights.data_ptr(), 1 if weigh_output else 0, x.data_ptr(), x.stride(0), 1 if accumulate else 0, n, top, width, ff, _stream())
     return x
+
+
+def routed_experts(h, w_gate, w_up, w_down, ids, weights, x, accumulate=True, weigh="input", activation="silu"):
+    """x[row] (+)= sum over the row's choices of expert(a): the whole mixture behind the router's choice.  weigh "input": a = weight * h[row]
+    (stored as h's dtype); "output": a = h[row] and the weight multiplies the expert's result."""
+    if weigh not in ("input", "output"):
+        raise KernelError(f"routed_experts: the weights weigh an expert's 'input' or its 'output', not {weigh!r}")
+    n, top = ids.shape
+    mid_dtype = torch.float32 if w_down.dtype == torch.float32 else h.dtype
+    mid = torch.empty((n * top, w_gate.shape[1]), dtype=mid_dtype, device=h.device)
+    experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=weigh == "input", activation=activation)
+    experts_down(mid, w_down, ids, weights, x, accumulate=accumulate, weigh_output=weigh == "output")
+    return x
+

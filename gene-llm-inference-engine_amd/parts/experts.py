@@ -66,9 +66,7 @@ class RoutedExperts(FeedForward):
         ids = torch.empty((T, s.top), dtype=torch.int32, device=dev)
         weights = torch.empty((T, s.top), dtype=torch.float32, device=dev)
         ops.route_top(logits, s.top, ids, weights, s.score, s.renormalize)
-        mid = torch.empty((T * s.top, s.intermediate_size), dtype=self.mid_dtype, device=dev)
-        ops.experts_gate_up(rows, self.w_gate, self.w_up, ids, weights, mid, weigh_input=s.weigh == "input", activation=s.activation)
-        ops.experts_down(mid, self.w_down, ids, weights, residual, accumulate=not overwrite, weigh_output=s.weigh == "output")
+        ops.routed_experts(rows, self.w_gate, self.w_up, self.w_down, ids, weights, residual, accumulate=not overwrite, weigh=s.weigh, activation=s.activation)
         if self.shared is not None:
             self.shared.forward(rows, residual, ctx)
         return None
