@@ -343,10 +343,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
 constexpr int PK = 64;
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+// (`tile_m`: which tile of BM rows the workgroup makes; blockIdx.x and .z say which columns and which share of k.)
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int EPI>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                             int M, int N, int K, long lda, long ldw, long ldc, int k_per_split,
-                                                             long split_stride, NormIn norm_in, RopeStore rope, NormOut norm_out) {
+__device__ __forceinline__ void piped_tile(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C, int M, int N, int K, long lda,
+                                           long ldw, long ldc, int k_per_split, long split_stride, const NormIn& norm_in, const RopeStore& rope,
+                                           const NormOut& norm_out, const int tile_m) {
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N, TM = WM / 32, TN = WN / 32;
     constexpr int ROWS = BM + BN, STAGE_BYTES = ROWS * 128, LOADS = ROWS / 8 / (WAVES_M * WAVES_N);      // loads per wave and stage
     static_assert(ROWS % (8 * WAVES_M * WAVES_N) == 0, "the rows of a stage must divide among the waves' loads");
@@ -354,7 +355,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
     extern __shared__ __attribute__((aligned(16))) unsigned char ring[];               // STAGES * STAGE_BYTES
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = (wave / WAVES_N) * WM, wn = (wave % WAVES_N) * WN;
-    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int m0 = tile_m * BM, n0 = blockIdx.x * BN;
 
     const bf16_t* src[LOADS];                  // this lane's source of each of its wave's loads, at k = 0
 #pragma unroll
@@ -505,6 +506,27 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
                     if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
                 }
             }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int EPI>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
+                                                             int M, int N, int K, long lda, long ldw, long ldc, int k_per_split,
+                                                             long split_stride, NormIn norm_in, RopeStore rope, NormOut norm_out) {
+    piped_tile<BM, BN, WAVES_M, WAVES_N, STAGES, EPI>(A, W, C, M, N, K, lda, ldw, ldc, k_per_split, split_stride, norm_in, rope, norm_out, blockIdx.y);
+}
+
+// The same tiles for many matrices at once: the rows of A lie in runs of whole tiles of 128, every run multiplied by its own
+// matrix W + group * group_stride; `tile_group` [tiles] names every tile's matrix (negative: the tile is not in use).  Rows that
+// fill up a run's last tile hold anything; their results are stored like the others and nobody reads them.
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_grouped_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C, int M, int N,
+                                                               int K, long lda, long ldw, long ldc, const int* __restrict__ tile_group, long group_stride) {
+    const int g = tile_group[blockIdx.y];
+    if (g < 0) return;
+    const NormIn no_norm_in = {nullptr, 0, 0.f, 1};
+    const NormOut no_norm_out = {nullptr, nullptr, 0, nullptr};
+    const RopeStore no_rope = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, 0};
+    piped_tile<128, 128, 2, 2, 2, EPI>(A, W + (size_t)g * group_stride, C, M, N, K, lda, ldw, ldc, K, 0L, no_norm_in, no_rope, no_norm_out, blockIdx.y);
 }
 
 // --------------------------------------------------------------------------------------- pingpong
@@ -1901,5 +1923,40 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     }
 #undef TILED
     GI_CHECK_LAUNCH("gemm_bf16 (tiled)");
+    return 0;
+}
+
+// C[rows of tile t] = A[rows of tile t] * W[tile_group[t]]^T for every tile t of 128 rows of A that is in use (see the kernel).  M rows
+// of A and C exist (a multiple of 128); W is [groups][N][K].  Output: float32 stored, bfloat16 stored, or the gated form.
+GI_API int gi_gemm_bf16_grouped(const void* A, const void* W, void* C, int c_dtype, int gated, int M, int N, int K, long lda, long ldw, long ldc,
+                                const int* tile_group, long group_stride, hipStream_t stream) {
+    GI_REQUIRE(M > 0 && M % 128 == 0 && N >= 128 && K > 0 && K % PK == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= (gated ? N / 2 : N)
+               && group_stride % 8 == 0 && M / 128 <= 65535,
+               "gemm_bf16_grouped: M %d (a multiple of 128), N %d (128 or more), K %d (a multiple of %d) or the strides do not fit", M, N, K, PK);
+    GI_REQUIRE(((uintptr_t)A & 15) == 0 && ((uintptr_t)W & 15) == 0, "gemm_bf16_grouped: operands must be 16-byte aligned");
+    int epi = epilogue_of(c_dtype, 0);
+    if (gated) {
+        GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16, "gemm_bf16_grouped: the gated product needs N %% 32 == 0 and a bfloat16 output");
+        epi = gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
+    }
+    GI_REQUIRE(epi >= 0, "gemm_bf16_grouped: output dtype %d is not supported", c_dtype);
+    constexpr int bytes = 2 * 256 * 128;
+    dim3 grid((N + 127) / 128, M / 128);
+#define GROUPED(EPI_)                                                                                                                               \
+    do {                                                                                                                                            \
+        static bool raised = false;                                                                                                                 \
+        if (!raised) {                                                                                                                              \
+            if (hipFuncSetAttribute((const void*)gemm_bf16_grouped_kernel<EPI_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) \
+                return gi_fail("gemm_bf16_grouped: cannot reserve %d bytes of LDS", bytes);                                                         \
+            raised = true;                                                                                                                          \
+        }                                                                                                                                           \
+        gemm_bf16_grouped_kernel<EPI_><<<grid, 256, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, tile_group, group_stride); \
+    } while (0)
+    if (epi == EPI_STORE_F32) GROUPED(EPI_STORE_F32);
+    else if (epi == EPI_STORE_BF16) GROUPED(EPI_STORE_BF16);
+    else if (epi == EPI_GATED_BF16) GROUPED(EPI_GATED_BF16);
+    else GROUPED(EPI_GATED_GELU_BF16);
+#undef GROUPED
+    GI_CHECK_LAUNCH("gemm_bf16 (grouped)");
     return 0;
 }

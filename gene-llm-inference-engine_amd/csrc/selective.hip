@@ -78,8 +78,16 @@ __global__ __launch_bounds__(256) void ssm_tail_kernel(const float* __restrict__
 }
 
 // The recurrence: one wave per (request of the step, 16 channels).  lane = channel * 4 + part; a lane keeps the states part,
-// part + 4, ... of its channel (NPL of them at most).
-template <int NPL, typename TO>
+// part + 4, ... of its channel (NPL of them at most).  The rows are taken RB at a time: the inputs of the next RB rows are asked
+// for, all at once, before the RB rows at hand are stepped through, and what does not depend on the state (step sizes, the gate's
+// SiLU) is made for all of them first, so that between two rows only the state's own multiply-add waits for the row before.
+// QUICK: exponentials by the hardware's exp2 (the results leave as bfloat16).
+template <int RB, int NPL>
+struct ScanRows {
+    float x[RB], dt[RB], z[RB], B[RB][NPL], C[RB][NPL];
+};
+
+template <int NPL, int RB, bool QUICK, typename TO>
 __global__ __launch_bounds__(64) void ssm_scan_kernel(const float* __restrict__ x, const float* __restrict__ dt_pre, long ld_dt, const float* __restrict__ dt_bias,
                                                      const float* __restrict__ bc, long ld_bc, int b_off, int c_off, const float* __restrict__ z, long ld_z,
                                                      const float* __restrict__ a_log, const float* __restrict__ d_skip, const int* __restrict__ seg_start,
@@ -98,41 +106,52 @@ __global__ __launch_bounds__(64) void ssm_scan_kernel(const float* __restrict__ 
         const int n = part + 4 * i;
         S[i] = n < n_state ? mine[n] : 0.f;
         A[i] = n < n_state ? -expf(a_log[(size_t)cc * n_state + n]) : 0.f;
+        if (QUICK) A[i] *= 1.4426950408889634f;
     }
     const float bias = dt_bias[cc], skip = d_skip[cc];
-    float xv = x[(size_t)t0 * inner + cc], pre = dt_pre[(size_t)t0 * ld_dt + cc], zv = z[(size_t)t0 * ld_z + cc];
-    float B[NPL], C[NPL];
+    auto ask = [&](ScanRows<RB, NPL>& rows, int r0) {
 #pragma unroll
-    for (int i = 0; i < NPL; ++i) {
-        const int n = min(part + 4 * i, n_state - 1);
-        B[i] = bc[(size_t)t0 * ld_bc + b_off + n];
-        C[i] = bc[(size_t)t0 * ld_bc + c_off + n];
-    }
-    for (int r = 0; r < n_rows; ++r) {
-        const int t = t0 + r, tn = t0 + min(r + 1, n_rows - 1);      // the next row's inputs are asked for now (the last row asks for itself again)
-        const float nx = x[(size_t)tn * inner + cc], npre = dt_pre[(size_t)tn * ld_dt + cc], nz = z[(size_t)tn * ld_z + cc];
-        float nB[NPL], nC[NPL];
+        for (int j = 0; j < RB; ++j) {
+            const size_t t = t0 + min(r0 + j, n_rows - 1);          // (rows behind the last ask for the last again)
+            rows.x[j] = x[t * inner + cc];
+            rows.dt[j] = dt_pre[t * ld_dt + cc];
+            rows.z[j] = z[t * ld_z + cc];
 #pragma unroll
-        for (int i = 0; i < NPL; ++i) {
-            const int n = min(part + 4 * i, n_state - 1);
-            nB[i] = bc[(size_t)tn * ld_bc + b_off + n];
-            nC[i] = bc[(size_t)tn * ld_bc + c_off + n];
-        }
-        const float dt = softplus_f(pre + bias), dx = dt * xv;
-        float acc = 0.f;
-#pragma unroll
-        for (int i = 0; i < NPL; ++i) {
-            if (part + 4 * i < n_state) {
-                S[i] = fmaf(expf(dt * A[i]), S[i], dx * B[i]);
-                acc = fmaf(S[i], C[i], acc);
+            for (int i = 0; i < NPL; ++i) {
+                const int n = min(part + 4 * i, n_state - 1);
+                rows.B[j][i] = bc[t * ld_bc + b_off + n];
+                rows.C[j][i] = bc[t * ld_bc + c_off + n];
             }
         }
-        acc += __shfl_xor(acc, 1, 64);
-        acc += __shfl_xor(acc, 2, 64);
-        if (live && part == 0) store_f32(out, (size_t)t * ldo + c, fmaf(skip, xv, acc) * silu_f(zv));
-        xv = nx, pre = npre, zv = nz;
+    };
+    ScanRows<RB, NPL> now, next;
+    ask(now, 0);
+    for (int r0 = 0; r0 < n_rows; r0 += RB) {
+        if (r0 + RB < n_rows) ask(next, r0 + RB);
 #pragma unroll
-        for (int i = 0; i < NPL; ++i) B[i] = nB[i], C[i] = nC[i];
+        for (int j = 0; j < RB; ++j) {
+            now.dt[j] = softplus_f(now.dt[j] + bias);
+            now.z[j] = silu_f(now.z[j]);
+        }
+#pragma unroll
+        for (int j = 0; j < RB; ++j) {
+            if (r0 + j < n_rows) {
+                const float dt = now.dt[j], dx = dt * now.x[j];
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < NPL; ++i) {
+                    if (part + 4 * i < n_state) {
+                        const float decay = QUICK ? __builtin_amdgcn_exp2f(dt * A[i]) : expf(dt * A[i]);
+                        S[i] = fmaf(decay, S[i], dx * now.B[j][i]);
+                        acc = fmaf(S[i], now.C[j][i], acc);
+                    }
+                }
+                acc += __shfl_xor(acc, 1, 64);
+                acc += __shfl_xor(acc, 2, 64);
+                if (live && part == 0) store_f32(out, (size_t)(t0 + r0 + j) * ldo + c, fmaf(skip, now.x[j], acc) * now.z[j]);
+            }
+        }
+        if (r0 + RB < n_rows) now = next;
     }
     if (live) {
 #pragma unroll
@@ -182,19 +201,19 @@ GI_API int gi_ssm_scan(const float* x, const float* dt_pre, long ld_dt, const fl
                "ssm_scan: bad sizes (requests %d, channels %d, states %d)", n_segs, inner, n_state);
     dim3 grid(n_segs, (inner + 15) / 16);
     GI_REQUIRE(grid.y <= 65535, "ssm_scan: too many channels");
-#define LAUNCH(NPL, TO)                                                                                                                            \
-    ssm_scan_kernel<NPL, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, seg_len, \
-                                                      row_slot, state, state_stride, (TO*)out, ldo, inner, n_state)
-#define BY_STATES(TO)                                  \
-    do {                                               \
-        if (n_state <= 16) LAUNCH(4, TO);              \
-        else if (n_state <= 32) LAUNCH(8, TO);         \
-        else if (n_state <= 64) LAUNCH(16, TO);        \
-        else if (n_state <= 128) LAUNCH(32, TO);       \
-        else LAUNCH(64, TO);                           \
+#define LAUNCH(NPL, RB, QUICK, TO)                                                                                                                         \
+    ssm_scan_kernel<NPL, RB, QUICK, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, seg_len, \
+                                                                 row_slot, state, state_stride, (TO*)out, ldo, inner, n_state)
+#define BY_STATES(QUICK, TO)                                     \
+    do {                                                         \
+        if (n_state <= 16) LAUNCH(4, 16, QUICK, TO);             \
+        else if (n_state <= 32) LAUNCH(8, 8, QUICK, TO);         \
+        else if (n_state <= 64) LAUNCH(16, 4, QUICK, TO);        \
+        else if (n_state <= 128) LAUNCH(32, 2, QUICK, TO);       \
+        else LAUNCH(64, 1, QUICK, TO);                           \
     } while (0)
-    if (out_dtype == GI_F32) BY_STATES(float);
-    else if (out_dtype == GI_BF16) BY_STATES(bf16_t);
+    if (out_dtype == GI_F32) BY_STATES(false, float);
+    else if (out_dtype == GI_BF16) BY_STATES(true, bf16_t);
     else return gi_fail("ssm_scan: unknown dtype %d", out_dtype);
 #undef BY_STATES
 #undef LAUNCH

@@ -50,7 +50,12 @@ _SIGNATURES = {
     "gi_ssm_scan": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                     c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p],
     "gi_route_top": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
-    "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_route_rows": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
+    "gi_experts_place": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
+    "gi_experts_gather": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_void_p],
+    "gi_experts_combine": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_int, c_void_p],
+    "gi_gemm_bf16_grouped": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_experts_down": [c_void_p, c_int, c_long, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_xielu": [c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p, c_void_p],
     "gi_delta_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
@@ -1533,6 +1538,9 @@ def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start,
 # ------------------------------------------------------------------------------------------------------------------ routed experts
 ROUTER_SCORES = {"sigmoid": 0, "softmax": 1}
 ROUTER_MAX_EXPERTS, ROUTER_MAX_TOP = 1024, 64
+EXPERT_ROW_GROUP = 16          # rows of a group where an expert's gates and up products lie in one matrix (`interleave_gate_up`)
+EXPERT_TILE_ROWS = 128         # rows of a tile of the product for grouped rows (the library's gi_experts_tile_rows)
+EXPERTS_GROUPED_FROM = 8       # (row, choice) items from which the experts' rows are grouped for the matrix cores
 
 
 def route_top(logits, top, ids, weights, score="sigmoid", renormalize=False):
@@ -1557,18 +1565,24 @@ def _expert_stack(w, rows, cols, what):
 
 def experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=True, activation="silu"):
     """mid[(row, choice)] = act(W_gate[e] a) * (W_up[e] a), a = the row of h (times the choice's weight if `weigh_input`, stored as
-    h's dtype), e = ids[row, choice]; one wave per output, for the few rows of decoding steps."""
+    h's dtype), e = ids[row, choice]; one wave per output, for the few rows of decoding steps.  w_up None: w_gate is one stack
+    [experts, 2 ff, width] of 16 gate rows, the 16 up rows of the same outputs, and so on (`interleave_gate_up` per expert)."""
     _dev(h, w_gate, w_up, ids, weights, mid)
     n, width = h.shape
-    top, ff = ids.shape[1], w_gate.shape[1]
-    _expert_stack(w_gate, ff, width, "experts_gate_up: the gates")
-    _expert_stack(w_up, ff, width, "experts_gate_up: the up products")
-    if not (h.stride(1) == 1 and mid.shape == (n * top, ff) and mid.stride(1) == 1 and w_gate.dtype == w_up.dtype and ids.dtype == torch.int32 and ids.is_contiguous()
-            and ids.shape == (n, top) and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()):
+    top = ids.shape[1]
+    group = 0 if w_up is not None else EXPERT_ROW_GROUP
+    ff = w_gate.shape[1] if w_up is not None else w_gate.shape[1] // 2
+    _expert_stack(w_gate, ff if w_up is not None else 2 * ff, width, "experts_gate_up: the gates")
+    if w_up is not None:
+        _expert_stack(w_up, ff, width, "experts_gate_up: the up products")
+    elif ff % EXPERT_ROW_GROUP:
+        raise KernelError(f"experts_gate_up: gates and up products in one stack come in groups of {EXPERT_ROW_GROUP} rows")
+    if not (h.stride(1) == 1 and mid.shape == (n * top, ff) and mid.stride(1) == 1 and (w_up is None or w_gate.dtype == w_up.dtype) and ids.dtype == torch.int32
+            and ids.is_contiguous() and ids.shape == (n, top) and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()):
         raise KernelError("experts_gate_up: h [n, width], mid [n * top, ff], ids int32 and weights float32 [n, top] are needed")
-    _call("gi_experts_gate_up", h.data_ptr(), _code(h, "experts_gate_up: h"), h.stride(0), w_gate.data_ptr(), w_up.data_ptr(), _code(w_gate, "experts_gate_up: weights"),
+    _call("gi_experts_gate_up", h.data_ptr(), _code(h, "experts_gate_up: h"), h.stride(0), w_gate.data_ptr(), _ptr(w_up), _code(w_gate, "experts_gate_up: weights"),
           ids.data_ptr(), weights.data_ptr(), 1 if weigh_input else 0, mid.data_ptr(), _code(mid, "experts_gate_up: mid"), mid.stride(0), n, top, width, ff,
-          ACTIVATIONS[activation], _stream())
+          ACTIVATIONS[activation], group, _stream())
     return mid
 
 
@@ -1587,15 +1601,89 @@ def experts_down(mid, w_down, ids, weights, x, accumulate=True, weigh_output=Fal
     return x
 
 
+def route_rows(h, router, top, ids, weights, score="sigmoid", renormalize=False, logits=None):
+    """The router's product and its choice in one launch: logits = h @ router.T with 32-bit sums in an order that the width alone
+    fixes, then as `route_top`.  logits: float32 [n, experts] to keep them in, or None."""
+    _dev(h, router, ids, weights, logits)
+    n, width = h.shape
+    n_experts = router.shape[0]
+    if score not in ROUTER_SCORES:
+        raise KernelError(f"route_rows: unknown score {score!r}; known: {', '.join(ROUTER_SCORES)}")
+    if not (1 <= top <= min(n_experts, ROUTER_MAX_TOP) and n_experts <= ROUTER_MAX_EXPERTS):
+        raise KernelError(f"route_rows: top {top} of {n_experts} experts is outside what the kernel takes")
+    if not (h.stride(1) == 1 and router.shape == (n_experts, width) and router.stride(1) == 1 and ids.dtype == torch.int32 and ids.shape == (n, top) and ids.is_contiguous()
+            and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()):
+        raise KernelError("route_rows: h [n, width], the router [experts, width], ids int32 and weights float32 [n, top] are needed")
+    if logits is not None:
+        _f32_rows(logits, "route_rows: logits", n, n_experts)
+    _call("gi_route_rows", h.data_ptr(), _code(h, "route_rows: h"), h.stride(0), router.data_ptr(), _code(router, "route_rows: the router"), router.stride(0), n, width,
+          n_experts, top, ROUTER_SCORES[score], 1 if renormalize else 0, ids.data_ptr(), weights.data_ptr(), _ptr(logits), logits.stride(0) if logits is not None else 0, _stream())
+
+
+def gemm_bf16_grouped(a, w, out, tile_group, gated=False):
+    """out[rows of tile t] = a[rows of tile t] @ w[tile_group[t]].T for every tile t of 128 rows with tile_group[t] >= 0: bfloat16 on
+    the matrix cores.  a [m, k] with m a multiple of 128, w [groups, n, k], out float32 or bfloat16 [m, n], or, gated (as
+    `gemm_bf16`), bfloat16 [m, n / 2].  Tiles with a negative entry are left as they are."""
+    _dev(a, w, out, tile_group)
+    m, k = a.shape
+    n = w.shape[1]
+    if not (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.dim() == 3 and w.shape[2] == k and w.is_contiguous() and a.stride(1) == 1 and out.stride(1) == 1
+            and out.shape == (m, n // 2 if gated else n) and m % EXPERT_TILE_ROWS == 0):
+        raise KernelError("gemm_bf16_grouped: a bfloat16 [m, k] (m a multiple of 128), w bfloat16 [groups, n, k] and out [m, n] (gated: [m, n / 2]) are needed")
+    _i32(tile_group, "gemm_bf16_grouped: the tiles' groups", m // EXPERT_TILE_ROWS)
+    if gated and gated is not True and gated not in ACTIVATIONS:
+        raise KernelError(f"gemm_bf16_grouped: unknown activation {gated!r} of a gated product")
+    gate_code = 0 if not gated else 1 + (0 if gated is True else ACTIVATIONS[gated])
+    if _profile is not None:
+        _profile.note = (f"{m}x{n}x{k}{' gated' if gated else ''}", 0)
+    _call("gi_gemm_bf16_grouped", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm_bf16_grouped: out"), gate_code, m, n, k, a.stride(0), w.stride(1),
+          out.stride(0), tile_group.data_ptr(), w.stride(0), _stream())
+    return out
+
+
+def experts_grouped_supported(h, w_gate, w_up, w_down) -> bool:
+    """Whether `routed_experts` can take many rows through the product for grouped rows: bfloat16 throughout, gates and up products
+    in one stack, and sizes the tiles take."""
+    if w_up is not None or not (h.dtype == w_gate.dtype == w_down.dtype == torch.bfloat16):
+        return False
+    width, ff = h.shape[1], w_down.shape[2]
+    return width % 64 == 0 and ff % 64 == 0 and width >= 128 and 2 * ff >= 128 and h.stride(0) % 8 == 0 and h.data_ptr() % 16 == 0
+
+
 def routed_experts(h, w_gate, w_up, w_down, ids, weights, x, accumulate=True, weigh="input", activation="silu"):
     """x[row] (+)= sum over the row's choices of expert(a): the whole mixture behind the router's choice.  weigh "input": a = weight * h[row]
-    (stored as h's dtype); "output": a = h[row] and the weight multiplies the expert's result."""
+    (stored as h's dtype); "output": a = h[row] and the weight multiplies the expert's result.  w_up None: w_gate holds both (see
+    `experts_gate_up`).  Few items, or 32-bit operands: every item walks its expert's matrices.  Many in bfloat16: the items' rows are
+    put in the order of their experts and all experts' products are two launches on the matrix cores."""
     if weigh not in ("input", "output"):
         raise KernelError(f"routed_experts: the weights weigh an expert's 'input' or its 'output', not {weigh!r}")
     n, top = ids.shape
+    n_experts, width = w_down.shape[0], w_down.shape[1]
+    ff = w_down.shape[2]
+    if n * top >= EXPERTS_GROUPED_FROM and experts_grouped_supported(h, w_gate, w_up, w_down):
+        _dev(h, w_gate, w_down, ids, weights, x)
+        _f32_rows(x, "routed_experts: x", n, width)
+        if not (ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()
+                and w_gate.shape == (n_experts, 2 * ff, width) and h.shape == (n, width)):
+            raise KernelError("routed_experts: ids int32 and weights float32 [n, top], gates and up products [experts, 2 ff, width] are needed")
+        tile = EXPERT_TILE_ROWS
+        n_tiles = max(1, (n * top + n_experts * (tile - 1)) // tile)
+        dev = h.device
+        book = torch.empty(n_experts + n * top + n_tiles, dtype=torch.int32, device=dev)
+        count, place, tile_expert = book[:n_experts], book[n_experts:n_experts + n * top], book[n_experts + n * top:]
+        _call("gi_experts_place", ids.data_ptr(), n * top, n_experts, count.data_ptr(), place.data_ptr(), tile_expert.data_ptr(), n_tiles, _stream())
+        rows = torch.empty((n_tiles * tile, width), dtype=torch.bfloat16, device=dev)
+        _call("gi_experts_gather", h.data_ptr(), h.stride(0), place.data_ptr(), weights.data_ptr(), 1 if weigh == "input" else 0, n, top, rows.data_ptr(), rows.stride(0),
+              width, _stream())
+        mid = torch.empty((n_tiles * tile, ff), dtype=torch.bfloat16, device=dev)
+        gemm_bf16_grouped(rows, w_gate, mid, tile_expert, gated=True if activation == "silu" else activation)
+        y = torch.empty((n_tiles * tile, width), dtype=torch.float32, device=dev)
+        gemm_bf16_grouped(mid, w_down, y, tile_expert)
+        _call("gi_experts_combine", y.data_ptr(), y.stride(0), place.data_ptr(), weights.data_ptr(), 1 if weigh == "output" else 0, n, top, x.data_ptr(), x.stride(0),
+              width, 1 if accumulate else 0, _stream())
+        return x
     mid_dtype = torch.float32 if w_down.dtype == torch.float32 else h.dtype
-    mid = torch.empty((n * top, w_gate.shape[1]), dtype=mid_dtype, device=h.device)
+    mid = torch.empty((n * top, ff), dtype=mid_dtype, device=h.device)
     experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=weigh == "input", activation=activation)
     experts_down(mid, w_down, ids, weights, x, accumulate=accumulate, weigh_output=weigh == "output")
     return x
-

@@ -1,9 +1,11 @@
 """A mixture of gated feed-forwards behind a router (`config.spec.RoutedExpertsSpec` states the rules; kernels: `csrc/experts.hip`).
 
-The router's logits are a 32-bit product of the normed rows (as the compute dtype stores them) with the router's matrix; one
-kernel turns them into every row's choice of experts and their weights.  The experts' matrices lie in three stacks
-[experts, ...], and every (row, choice) walks its own expert's: nothing of a step's shape depends on the router's choices, so a
-captured pass may contain the part.  A shared feed-forward, if the spec names one, is a part of its own kind and adds onto the
+The router's logits are a 32-bit product of the normed rows (as the compute dtype stores them) with the router's matrix; the
+same kernel turns them into every row's choice of experts and their weights.  The experts' matrices lie in stacks
+[experts, ...] (in bfloat16 an expert's gates and up products interleaved in one matrix, for the product with the gate inside).
+A few (row, choice) items walk their own expert's matrices each; many are put in the order of their experts on the device and
+go through the matrix cores, all experts in one launch.  Either way nothing of a step's shape depends on the router's choices,
+so a captured pass may contain the part.  A shared feed-forward, if the spec names one, is a part of its own kind and adds onto the
 same rows."""
 from __future__ import annotations
 
@@ -32,9 +34,14 @@ class RoutedExperts(FeedForward):
         if s.n_experts > ops.ROUTER_MAX_EXPERTS or s.top > ops.ROUTER_MAX_TOP:
             raise ValueError(f"routed experts: at most {ops.ROUTER_MAX_EXPERTS} experts and {ops.ROUTER_MAX_TOP} a row")
         self.router = tensors[s.router]
-        self.w_gate = torch.stack([tensors[n] for n in s.gate_projs]).contiguous()
-        self.w_up = torch.stack([tensors[n] for n in s.up_projs]).contiguous()
         self.w_down = torch.stack([tensors[n] for n in s.down_projs]).contiguous()
+        if self.w_down.dtype == torch.bfloat16 and dtype == torch.bfloat16 and s.intermediate_size % ops.EXPERT_ROW_GROUP == 0:
+            # gates and up products in one stack, as the product with the gate inside reads them
+            self.w_gate = torch.stack([ops.interleave_gate_up(tensors[g], tensors[u]) for g, u in zip(s.gate_projs, s.up_projs)]).contiguous()
+            self.w_up = None
+        else:
+            self.w_gate = torch.stack([tensors[n] for n in s.gate_projs]).contiguous()
+            self.w_up = torch.stack([tensors[n] for n in s.up_projs]).contiguous()
         self.in_dtype = activation_dtype_for(self.w_gate, dtype)
         self.mid_dtype = activation_dtype_for(self.w_down, dtype)
         self.shared = None if s.shared is None else feed_forward_class(s.shared)(s.shared, tensors, dtype, device)
@@ -55,17 +62,15 @@ class RoutedExperts(FeedForward):
     def weights_read_per_step(self):
         """What a step of few rows reads: the router, `top` experts a row at most (here: of one row), the shared feed-forward."""
         s = self.spec
-        share = [w[:min(s.top, s.n_experts)] for w in (self.w_gate, self.w_up, self.w_down)]
+        share = [w[:min(s.top, s.n_experts)] for w in (self.w_gate, self.w_up, self.w_down) if w is not None]
         return [self.router, *share] + ([self.shared] if self.shared is not None else [])
 
     def forward(self, h, residual, ctx, then=None, overwrite=False):
         s, T, dev = self.spec, ctx.n_rows, ctx.device
         rows = h.materialize() if isinstance(h, NormedRows) else h
-        logits = torch.empty((T, s.n_experts), dtype=torch.float32, device=dev)
-        ops.gemm_exact(rows, self.router, logits)
         ids = torch.empty((T, s.top), dtype=torch.int32, device=dev)
         weights = torch.empty((T, s.top), dtype=torch.float32, device=dev)
-        ops.route_top(logits, s.top, ids, weights, s.score, s.renormalize)
+        ops.route_rows(rows, self.router, s.top, ids, weights, s.score, s.renormalize)
         ops.routed_experts(rows, self.w_gate, self.w_up, self.w_down, ids, weights, residual, accumulate=not overwrite, weigh=s.weigh, activation=s.activation)
         if self.shared is not None:
             self.shared.forward(rows, residual, ctx)

@@ -152,6 +152,12 @@ def test_selective_scan_kernels(inner, N, taps):
         both = run(slice(0, k), portion, [1, 3], [lens[0], lens[1]])[1]
         alone = torch.cat([run(slice(0, portion[0]), [portion[0]], [2], [lens[0]])[1], run(slice(portion[0], k), [portion[1]], [4], [lens[1]])[1]])
         assert torch.equal(both, alone) and torch.equal(state[1], state[2]) and torch.equal(state[3], state[4])
+    # results stored as bfloat16 (the kernel's quick exponentials): as close as their 8 bits allow
+    state[1] = 0
+    seg_start, seg_len, row_slot, row_pos = _segs([lens[0]], [1], [0])
+    half = torch.empty(lens[0], inner, device=DEV, dtype=torch.bfloat16)
+    ops.ssm_scan(dev(x1.float()), dev(dt_pre[first]), d_db, dev(low[first]), 2, 2 + N, dev(z[first]), d_al, d_D, seg_start, seg_len, row_slot, state, half, N)
+    assert relative_error(half, y1) < 4e-3 and relative_error(state[1, :inner * N].view(inner, N), S1) < 3e-5
     low_copy = torch.empty(5, inner, device=DEV, dtype=torch.bfloat16)
     seg_start, seg_len, row_slot, row_pos = _segs([5], [1], [0])
     state[1] = 0
@@ -178,10 +184,22 @@ def test_the_router_s_choice(experts, top):
         ids, weights = torch.empty(50, top, dtype=torch.int32, device=DEV), torch.empty(50, top, device=DEV)
         ops.route_top(logits.to(DEV)[:, :experts], top, ids, weights, score, renorm)
         assert torch.equal(ids.cpu().long(), order) and relative_error(weights, want) < 1e-6
+    # the product and the choice in one launch: the same choice from the same logits, whatever rows lie beside a row
+    for dtype in (torch.float32, torch.bfloat16):
+        h, router = torch.randn(50, 72, generator=g).to(dtype), torch.randn(experts, 72, generator=g).to(dtype)
+        ids2, weights2, kept = torch.empty_like(ids), torch.empty_like(weights), torch.empty(50, experts, device=DEV)
+        ops.route_rows(h.to(DEV), router.to(DEV), top, ids2, weights2, "softmax", True, logits=kept)
+        assert relative_error(kept, h.double() @ router.double().T) < 1e-6
+        ops.route_top(kept, top, ids, weights, "softmax", True)
+        assert torch.equal(ids, ids2) and torch.equal(weights, weights2)
+        one_i, one_w = torch.empty(1, top, dtype=torch.int32, device=DEV), torch.empty(1, top, device=DEV)
+        ops.route_rows(h.to(DEV)[17:18], router.to(DEV), top, one_i, one_w, "softmax", True)
+        assert torch.equal(one_i[0], ids2[17]) and torch.equal(one_w[0], weights2[17])
 
 
 @pytest.mark.parametrize("rows, d, ff, E, top, dtype", [(7, 50, 10, 3, 3, "float32"), (1, 64, 24, 5, 2, "float32"), (33, 128, 64, 8, 2, "bfloat16"), (300, 64, 48, 6, 1, "float32"),
-                                                        (150, 256, 96, 4, 2, "bfloat16"), (65, 40, 130, 9, 4, "float32")])
+                                                        (150, 256, 96, 4, 2, "bfloat16"), (65, 40, 130, 9, 4, "float32"), (300, 128, 128, 16, 4, "bfloat16"),
+                                                        (5, 192, 64, 3, 2, "bfloat16"), (2, 128, 64, 4, 2, "bfloat16"), (700, 192, 320, 5, 1, "bfloat16")])
 def test_routed_experts_against_the_plain_statement(rows, d, ff, E, top, dtype):
     """Few rows and many (every expert's rows together), the score on an expert's input or on its output; the second time onto rows
     that hold something."""
@@ -202,17 +220,21 @@ def test_routed_experts_against_the_plain_statement(rows, d, ff, E, top, dtype):
     ids, weights = torch.empty(rows, top, dtype=torch.int32, device=DEV), torch.empty(rows, top, device=DEV)
     ops.route_top(dev(logits), top, ids, weights)
     tol = 2e-2 if dtype == "bfloat16" else 3e-5
+    d_h, d_wg, d_wu, d_wd = dev(h), dev(wg), dev(wu), dev(wd)
+    if dtype == "bfloat16":           # as the part keeps them: an expert's gates and up products in one matrix
+        d_wg, d_wu = torch.stack([ops.interleave_gate_up(d_wg[e], d_wu[e]) for e in range(E)]).contiguous(), None
+        assert ops.experts_grouped_supported(d_h, d_wg, d_wu, d_wd) == (ff % 64 == 0)
     for weigh, want in (("input", want_in), ("output", want_out)):
         x = torch.full((rows, d), 0.5, device=DEV)
-        ops.routed_experts(dev(h), dev(wg), dev(wu), dev(wd), ids, weights, x, accumulate=True, weigh=weigh)
+        ops.routed_experts(d_h, d_wg, d_wu, d_wd, ids, weights, x, accumulate=True, weigh=weigh)
         assert relative_error(x - 0.5, want) < tol, weigh
         y = torch.full((rows, d), 7.0, device=DEV)
-        ops.routed_experts(dev(h), dev(wg), dev(wu), dev(wd), ids, weights, y, accumulate=False, weigh=weigh)
+        ops.routed_experts(d_h, d_wg, d_wu, d_wd, ids, weights, y, accumulate=False, weigh=weigh)
         assert relative_error(y, want) < tol
         if rows > 1:                                                      # a row's result does not depend on the rows beside it
             k = rows // 2
             alone = torch.zeros(1, d, device=DEV)
-            ops.routed_experts(dev(h)[k:k + 1], dev(wg), dev(wu), dev(wd), ids[k:k + 1].contiguous(), weights[k:k + 1].contiguous(), alone, accumulate=False, weigh=weigh)
+            ops.routed_experts(d_h[k:k + 1], d_wg, d_wu, d_wd, ids[k:k + 1].contiguous(), weights[k:k + 1].contiguous(), alone, accumulate=False, weigh=weigh)
             if dtype == "float32":
                 assert relative_error(alone[0], y[k]) < 1e-6
             else:
