@@ -10,6 +10,8 @@
 // worked on.
 //
 // State of one request slot, 32-bit: S [channels][states], then the convolution's last taps - 1 inputs [taps - 1][channels].
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -18,6 +20,17 @@ constexpr int SSM_MAX_TAPS = 8;
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+// The same two by the hardware's exp2, log2 and reciprocal (each within a unit or two in the last place of 32 bits), for results
+// that leave as bfloat16.
+__device__ __forceinline__ float silu_quick(float z) { return z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -1.4426950408889634f)); }
+__device__ __forceinline__ float softplus_quick(float z) {
+    return z > 20.f ? z : 0.6931471805599453f * __builtin_amdgcn_logf(1.0f + __builtin_amdgcn_exp2f(z * 1.4426950408889634f));
+}
+// The value of the lane that the quad permutation CTRL names (within groups of four lanes).
+template <int CTRL>
+__device__ __forceinline__ float quad_moved(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, false));
+}
 
 // How many of the rows t-1, t-2, ... (at most `most`) belong to the same request as row t and directly precede it.
 __device__ __forceinline__ int rows_before(const int* __restrict__ slot, const int* __restrict__ pos, int t, int most) {
@@ -87,77 +100,169 @@ struct ScanRows {
     float x[RB], dt[RB], z[RB], B[RB][NPL], C[RB][NPL];
 };
 
-template <int NPL, int RB, bool QUICK, typename TO>
+// PHASE 0: a workgroup takes a request's rows of the step from the request's state to its state.  Long runs of rows whose results
+// leave as bfloat16 are cut into chunks of `chunk_rows` rows instead, which all run at once:
+//   PHASE 1  every chunk but a request's last, from a zero state: where the chunk alone takes the state (`ends` [chunks][channels]
+//            [states]) and the sum of its step sizes (`sums` [chunks][channels]); nothing else is stored
+//   (ssm_carry_kernel: the state every chunk starts from, chunk after chunk: S <- exp(A * sum) S + end, into `ends`)
+//   PHASE 2  every chunk from the state it starts from, with the results; a request's last chunk leaves the request's state.
+// The sums of a row are taken in another order than from row to row: the results differ by 32-bit rounding.
+struct ScanChunk {
+    int t0, n_rows, index, last;      // first row, rows, the chunk's number in the step, whether it is its request's last
+};
+__device__ __forceinline__ bool find_chunk(ScanChunk& ch, int g, const int* __restrict__ seg_start, const int* __restrict__ seg_len, int n_segs, int chunk_rows) {
+    ch.index = g;
+    for (int s = 0; s < n_segs; ++s) {
+        const int rows = seg_len[s], chunks = (rows + chunk_rows - 1) / chunk_rows;
+        if (g < chunks) {
+            ch.t0 = seg_start[s] + g * chunk_rows;
+            ch.n_rows = min(chunk_rows, rows - g * chunk_rows);
+            ch.last = g == chunks - 1;
+            return true;
+        }
+        g -= chunks;
+    }
+    return false;
+}
+
+template <int NPL, int RB, bool QUICK, int PHASE, typename TO>
 __global__ __launch_bounds__(64) void ssm_scan_kernel(const float* __restrict__ x, const float* __restrict__ dt_pre, long ld_dt, const float* __restrict__ dt_bias,
                                                      const float* __restrict__ bc, long ld_bc, int b_off, int c_off, const float* __restrict__ z, long ld_z,
                                                      const float* __restrict__ a_log, const float* __restrict__ d_skip, const int* __restrict__ seg_start,
                                                      const int* __restrict__ seg_len, const int* __restrict__ row_slot, float* __restrict__ state,
-                                                     long state_stride, TO* __restrict__ out, long ldo, int inner, int n_state) {
-    const int n_rows = seg_len[blockIdx.x];
+                                                     long state_stride, TO* __restrict__ out, long ldo, int inner, int n_state, int n_segs, int chunk_rows,
+                                                     float* __restrict__ ends, float* __restrict__ sums) {
+    ScanChunk ch;
+    if (PHASE == 0) {
+        ch.t0 = seg_start[blockIdx.x], ch.n_rows = seg_len[blockIdx.x], ch.index = 0, ch.last = 1;
+    } else if (!find_chunk(ch, blockIdx.x, seg_start, seg_len, n_segs, chunk_rows) || (PHASE == 1 && ch.last)) {
+        return;
+    }
+    const int n_rows = ch.n_rows;
     if (n_rows <= 0) return;
-    const int t0 = seg_start[blockIdx.x], lane = threadIdx.x, part = lane & 3;
+    const int t0 = ch.t0, lane = threadIdx.x, part = lane & 3;
     const int c = blockIdx.y * 16 + (lane >> 2);
     const bool live = c < inner;
     const int cc = live ? c : inner - 1;                          // (idle lanes walk along on the last channel and store nothing)
     float* mine = state + (size_t)row_slot[t0] * state_stride + (size_t)cc * n_state;
+    float* my_end = PHASE == 0 ? nullptr : ends + ((size_t)ch.index * inner + cc) * n_state;
+    const float* from = PHASE == 0 ? mine : my_end;
     float S[NPL], A[NPL];
 #pragma unroll
     for (int i = 0; i < NPL; ++i) {
         const int n = part + 4 * i;
-        S[i] = n < n_state ? mine[n] : 0.f;
+        S[i] = PHASE != 1 && n < n_state ? from[n] : 0.f;
         A[i] = n < n_state ? -expf(a_log[(size_t)cc * n_state + n]) : 0.f;
         if (QUICK) A[i] *= 1.4426950408889634f;
     }
     const float bias = dt_bias[cc], skip = d_skip[cc];
+    float dt_sum = 0.f;
     auto ask = [&](ScanRows<RB, NPL>& rows, int r0) {
 #pragma unroll
         for (int j = 0; j < RB; ++j) {
             const size_t t = t0 + min(r0 + j, n_rows - 1);          // (rows behind the last ask for the last again)
             rows.x[j] = x[t * inner + cc];
             rows.dt[j] = dt_pre[t * ld_dt + cc];
-            rows.z[j] = z[t * ld_z + cc];
+            if (PHASE != 1) rows.z[j] = z[t * ld_z + cc];
 #pragma unroll
             for (int i = 0; i < NPL; ++i) {
                 const int n = min(part + 4 * i, n_state - 1);
                 rows.B[j][i] = bc[t * ld_bc + b_off + n];
-                rows.C[j][i] = bc[t * ld_bc + c_off + n];
+                if (PHASE != 1) rows.C[j][i] = bc[t * ld_bc + c_off + n];
             }
         }
     };
     ScanRows<RB, NPL> now, next;
     ask(now, 0);
-    for (int r0 = 0; r0 < n_rows; r0 += RB) {
-        if (r0 + RB < n_rows) ask(next, r0 + RB);
+    // The RB rows at hand.  What does not depend on the state comes first, for all rows: step sizes, the gate's SiLU, every state's
+    // decay and input.  Then the states step from row to row, one multiply-add each, and every row's read-out is summed over the
+    // channel's four lanes.  `whole`: all RB rows exist; otherwise the rows behind the last change nothing and are not stored.
+    auto step_rows = [&](int r0, auto whole) {
+        constexpr bool WHOLE = decltype(whole)::value;
+        float y[RB];
 #pragma unroll
         for (int j = 0; j < RB; ++j) {
-            now.dt[j] = softplus_f(now.dt[j] + bias);
-            now.z[j] = silu_f(now.z[j]);
+            now.dt[j] = QUICK ? softplus_quick(now.dt[j] + bias) : softplus_f(now.dt[j] + bias);
+            if (PHASE != 1) now.z[j] = QUICK ? silu_quick(now.z[j]) : silu_f(now.z[j]);
         }
 #pragma unroll
         for (int j = 0; j < RB; ++j) {
-            if (r0 + j < n_rows) {
-                const float dt = now.dt[j], dx = dt * now.x[j];
-                float acc = 0.f;
+            const bool valid = WHOLE || r0 + j < n_rows;
+            const float dt = now.dt[j], dx = dt * now.x[j];
+            float acc = 0.f;
 #pragma unroll
-                for (int i = 0; i < NPL; ++i) {
-                    if (part + 4 * i < n_state) {
-                        const float decay = QUICK ? __builtin_amdgcn_exp2f(dt * A[i]) : expf(dt * A[i]);
-                        S[i] = fmaf(decay, S[i], dx * now.B[j][i]);
-                        acc = fmaf(S[i], now.C[j][i], acc);
-                    }
-                }
-                acc += __shfl_xor(acc, 1, 64);
-                acc += __shfl_xor(acc, 2, 64);
-                if (live && part == 0) store_f32(out, (size_t)(t0 + r0 + j) * ldo + c, fmaf(skip, now.x[j], acc) * now.z[j]);
+            for (int i = 0; i < NPL; ++i) {
+                const float decay = QUICK ? __builtin_amdgcn_exp2f(dt * A[i]) : expf(dt * A[i]);
+                const float stepped = fmaf(decay, S[i], dx * now.B[j][i]);
+                S[i] = valid ? stepped : S[i];
+                if (PHASE != 1) acc = part + 4 * i < n_state ? fmaf(S[i], now.C[j][i], acc) : acc;
             }
+            if (PHASE == 1) {
+                dt_sum += valid ? dt : 0.f;
+                continue;
+            }
+            acc += quad_moved<0xB1>(acc);                          // lanes 1 apart: quad_perm [1, 0, 3, 2]
+            acc += quad_moved<0x4E>(acc);                          // lanes 2 apart: quad_perm [2, 3, 0, 1]
+            y[j] = fmaf(skip, now.x[j], acc) * now.z[j];
         }
-        if (r0 + RB < n_rows) now = next;
+        if (PHASE != 1 && live && part == 0) {
+#pragma unroll
+            for (int j = 0; j < RB; ++j)
+                if (WHOLE || r0 + j < n_rows) store_f32(out, (size_t)(t0 + r0 + j) * ldo + c, y[j]);
+        }
+    };
+    for (int r0 = 0; r0 < n_rows; r0 += RB) {
+        const bool more = r0 + RB < n_rows;
+        if (more) ask(next, r0 + RB);
+        if (r0 + RB <= n_rows) step_rows(r0, std::true_type{});
+        else step_rows(r0, std::false_type{});
+        if (more) now = next;
     }
-    if (live) {
+    if (PHASE == 1 && live && part == 0) sums[(size_t)ch.index * inner + c] = dt_sum;
+    float* to = PHASE == 1 ? my_end : mine;
+    if (live && (PHASE != 2 || ch.last)) {
 #pragma unroll
         for (int i = 0; i < NPL; ++i) {
             const int n = part + 4 * i;
-            if (n < n_state) mine[n] = S[i];
+            if (n < n_state) to[n] = S[i];
+        }
+    }
+}
+
+// Between the two phases: one wave per (request of the step, 16 channels) walks the request's chunks.  `ends` holds where every chunk
+// alone takes the state and gets the state the chunk starts from instead.
+template <int NPL, bool QUICK>
+__global__ __launch_bounds__(64) void ssm_carry_kernel(const float* __restrict__ a_log, const int* __restrict__ seg_start, const int* __restrict__ seg_len,
+                                                      const int* __restrict__ row_slot, const float* __restrict__ state, long state_stride, int inner, int n_state,
+                                                      int chunk_rows, float* __restrict__ ends, const float* __restrict__ sums) {
+    const int rows = seg_len[blockIdx.x];
+    if (rows <= 0) return;
+    int first = 0;
+    for (int s = 0; s < (int)blockIdx.x; ++s) first += (seg_len[s] + chunk_rows - 1) / chunk_rows;
+    const int chunks = (rows + chunk_rows - 1) / chunk_rows, lane = threadIdx.x, part = lane & 3;
+    const int c = blockIdx.y * 16 + (lane >> 2);
+    if (c >= inner) return;
+    const float* mine = state + (size_t)row_slot[seg_start[blockIdx.x]] * state_stride + (size_t)c * n_state;
+    float S[NPL], A[NPL];
+#pragma unroll
+    for (int i = 0; i < NPL; ++i) {
+        const int n = part + 4 * i;
+        S[i] = n < n_state ? mine[n] : 0.f;
+        A[i] = n < n_state ? -expf(a_log[(size_t)c * n_state + n]) : 0.f;
+        if (QUICK) A[i] *= 1.4426950408889634f;
+    }
+    for (int g = 0; g < chunks; ++g) {
+        float* at = ends + ((size_t)(first + g) * inner + c) * n_state;
+        const float sum = g + 1 < chunks ? sums[(size_t)(first + g) * inner + c] : 0.f;
+#pragma unroll
+        for (int i = 0; i < NPL; ++i) {
+            const int n = part + 4 * i;
+            if (n < n_state) {
+                const float end = g + 1 < chunks ? at[n] : 0.f;
+                at[n] = S[i];
+                const float decay = QUICK ? __builtin_amdgcn_exp2f(sum * A[i]) : expf(sum * A[i]);
+                S[i] = fmaf(decay, S[i], end);
+            }
         }
     }
 }
@@ -195,15 +300,29 @@ GI_API int gi_ssm_tail(const float* pre, long ld, int n_taps, const int* seg_sta
 
 GI_API int gi_ssm_scan(const float* x, const float* dt_pre, long ld_dt, const float* dt_bias, const float* bc, long ld_bc, int b_off, int c_off, const float* z,
                        long ld_z, const float* a_log, const float* d_skip, const int* seg_start, const int* seg_len, int n_segs, const int* row_slot,
-                       float* state, long state_stride, void* out, int out_dtype, long ldo, int inner, int n_state, hipStream_t stream) {
+                       float* state, long state_stride, void* out, int out_dtype, long ldo, int inner, int n_state, int n_chunks, int chunk_rows, float* ends,
+                       float* sums, hipStream_t stream) {
     GI_REQUIRE(n_segs > 0 && inner > 0 && n_state > 0 && n_state <= 256 && ld_dt >= inner && ld_z >= inner && ldo >= inner && b_off >= 0 && c_off >= 0
                && ld_bc >= b_off + n_state && ld_bc >= c_off + n_state && state_stride >= (long)inner * n_state,
                "ssm_scan: bad sizes (requests %d, channels %d, states %d)", n_segs, inner, n_state);
     dim3 grid(n_segs, (inner + 15) / 16);
     GI_REQUIRE(grid.y <= 65535, "ssm_scan: too many channels");
-#define LAUNCH(NPL, RB, QUICK, TO)                                                                                                                         \
-    ssm_scan_kernel<NPL, RB, QUICK, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, seg_len, \
-                                                                 row_slot, state, state_stride, (TO*)out, ldo, inner, n_state)
+    GI_REQUIRE(n_chunks == 0 || (n_chunks > 0 && chunk_rows > 0 && ends != nullptr && sums != nullptr && out_dtype == GI_BF16),
+               "ssm_scan: rows in chunks need the chunks' scratch memory and results stored as bfloat16");
+#define LAUNCH(NPL, RB, QUICK, TO)                                                                                                                            \
+    do {                                                                                                                                                      \
+        if (n_chunks == 0) {                                                                                                                                  \
+            ssm_scan_kernel<NPL, RB, QUICK, 0, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+                                                                            seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, 0, nullptr, nullptr); \
+        } else {                                                                                                                                              \
+            dim3 by_chunk(n_chunks, grid.y);                                                                                                                  \
+            ssm_scan_kernel<NPL, RB, QUICK, 1, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums); \
+            ssm_carry_kernel<NPL, QUICK><<<grid, 64, 0, stream>>>(a_log, seg_start, seg_len, row_slot, state, state_stride, inner, n_state, chunk_rows, ends, sums); \
+            ssm_scan_kernel<NPL, RB, QUICK, 2, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums); \
+        }                                                                                                                                                     \
+    } while (0)
 #define BY_STATES(QUICK, TO)                                     \
     do {                                                         \
         if (n_state <= 16) LAUNCH(4, 16, QUICK, TO);             \

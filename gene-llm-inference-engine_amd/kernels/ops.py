@@ -48,7 +48,7 @@ _SIGNATURES = {
     "gi_ssm_conv": [c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gi_ssm_tail": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p],
     "gi_ssm_scan": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                    c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p],
+                    c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "gi_route_top": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_route_rows": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
@@ -1511,10 +1511,18 @@ def ssm_tail(pre, n_taps, seg_start, seg_len, row_slot, state, inner, n_state):
           state.stride(0), inner, n_state, _stream())
 
 
-def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out, n_state):
+SSM_CHUNK_ROWS = 64            # rows of a chunk where a long run of rows is cut into chunks that run at once
+SSM_CHUNKS_FROM = 128          # rows of a step's longest request from which that is done
+
+
+def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out, n_state, rows_per_request=None):
     """The recurrence over every request's rows, from its state slot and back into it; out [n, inner] = (read-out + D x) * SiLU(z).
     x float32 [n, inner] contiguous; dt_pre, z float32 [n, inner] (any row stride); low float32 [n, >= offsets + n_state] holds B and
-    C of every row at the two offsets; dt_bias, d_skip float32 [inner]; a_log float32 [inner, n_state]."""
+    C of every row at the two offsets; dt_bias, d_skip float32 [inner]; a_log float32 [inner, n_state].
+    rows_per_request: the requests' numbers of rows as the host knows them (what seg_len holds).  Given, with results stored as
+    bfloat16 and a request of SSM_CHUNKS_FROM rows or more, the rows are cut into chunks of SSM_CHUNK_ROWS that run at once (every
+    chunk from a zero state first, then the states the chunks start from, then every chunk with its results): the same sums in
+    another order, so the results differ by 32-bit rounding from those of rows taken one after the other."""
     _dev(x, dt_pre, dt_bias, low, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out)
     n, inner = x.shape
     _f32_rows(dt_pre, "ssm_scan: the step sizes", n, inner)
@@ -1529,9 +1537,16 @@ def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start,
             raise KernelError(f"ssm_scan: {name} must be float32 {list(shape)}")
     _ssm_state(state, inner, n_state, 1, "ssm_scan")
     _i32(row_slot, "ssm_scan: slots", n)
+    n_chunks, ends, sums = 0, None, None
+    if rows_per_request is not None and out.dtype == torch.bfloat16 and max(rows_per_request) >= SSM_CHUNKS_FROM:
+        if len(rows_per_request) != seg_start.numel() or sum(rows_per_request) != n:
+            raise KernelError("ssm_scan: the requests' numbers of rows do not add up to the step's rows")
+        n_chunks = sum(-(-int(r) // SSM_CHUNK_ROWS) for r in rows_per_request)
+        ends = torch.empty((n_chunks, inner, n_state), dtype=torch.float32, device=x.device)
+        sums = torch.empty((n_chunks, inner), dtype=torch.float32, device=x.device)
     _call("gi_ssm_scan", x.data_ptr(), dt_pre.data_ptr(), dt_pre.stride(0), dt_bias.data_ptr(), low.data_ptr(), low.stride(0), int(b_off), int(c_off), z.data_ptr(),
           z.stride(0), a_log.data_ptr(), d_skip.data_ptr(), seg_start.data_ptr(), seg_len.data_ptr(), seg_start.numel(), row_slot.data_ptr(), state.data_ptr(),
-          state.stride(0), out.data_ptr(), _code(out, "ssm_scan: out"), out.stride(0), inner, n_state, _stream())
+          state.stride(0), out.data_ptr(), _code(out, "ssm_scan: out"), out.stride(0), inner, n_state, n_chunks, SSM_CHUNK_ROWS, _ptr(ends), _ptr(sums), _stream())
     return out
 
 

@@ -6,7 +6,8 @@ of single rows the kernel before it does that on its way).  A second product mak
 the channels' step sizes from dt.  One kernel steps the states over every request's rows, in order, from the request's state
 slot and back into it, and stores (read-out + D x) * SiLU(z) as the output product reads it.  The step sizes (from the third
 product on: bias, softplus), the decays and their exponentials, B, C, the state and the read-out are 32-bit, whatever the
-compute dtype.
+compute dtype.  In bfloat16 a request's long run of rows (a prompt) is cut into chunks that run at once (`ops.ssm_scan`); in
+float32 the rows are always taken one after the other, so that the bits do not depend on how a prompt was cut into steps.
 
 A request's state: S [inner][state] and the convolution's last taps - 1 inputs, one run of 32-bit numbers in the slot the
 cache manager gives it (zeroed when the request opens).  The runs of rows that belong to one request are found on the
@@ -92,7 +93,8 @@ class SelectiveScan(Mixer):
         dt_pre = torch.empty((T, inner), dtype=torch.float32, device=dev)
         linear(low[:, :R], self.w_dt, dt_pre)           # (32-bit rows: the step sizes' product keeps them)
         mid = torch.empty((T, inner), dtype=self.mid_dtype, device=dev)
-        ops.ssm_scan(x, dt_pre, self.dt_bias, low, R, R + N, z, self.a_log, self.d_skip, seg_start, seg_len, ctx.row_slot, cache.state, mid, N)
+        ops.ssm_scan(x, dt_pre, self.dt_bias, low, R, R + N, z, self.a_log, self.d_skip, seg_start, seg_len, ctx.row_slot, cache.state, mid, N,
+                     rows_per_request=ctx.seg_len)
         if overwrite:
             linear(mid, self.w_o, residual)
             return None

@@ -166,6 +166,50 @@ def test_selective_scan_kernels(inner, N, taps):
     assert torch.equal(low_copy.cpu(), xf.cpu().to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("inner, N, lens", [(40, 5, [300, 70, 129]), (72, 17, [128, 1, 64]), (16, 40, [513]), (33, 16, [2, 200, 191])])
+def test_selective_scan_of_long_runs_cut_into_chunks(inner, N, lens):
+    """Results stored as bfloat16, requests of a hundred rows and more beside short ones: the runs are cut into chunks that run at
+    once.  Every request starts from a state that holds something, and one channel barely decays, so that a chunk that started from
+    a wrong state would show in all rows behind it."""
+    from geneinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(inner + N)
+    n = sum(lens)
+    assert max(lens) >= ops.SSM_CHUNKS_FROM
+    x, z, dt_pre = torch.randn(n, inner, generator=g), torch.randn(n, inner, generator=g), torch.randn(n, inner, generator=g) - 1.0
+    low = torch.randn(n, 2 * N, generator=g)
+    a_log, dt_b, D = -0.5 + 0.6 * torch.randn(inner, N, generator=g), 0.5 * torch.randn(inner, generator=g), torch.randn(inner, generator=g)
+    a_log[0] = -9.0
+    slots = [3, 0, 2, 1][:len(lens)]
+    start = torch.randn(4, inner * N, generator=g)
+    want, ends, at = [], {}, 0
+    for m, slot in zip(lens, slots):
+        rows = slice(at, at + m)
+        dt = P.softplus(dt_pre[rows].double() + dt_b.double())
+        B, C, A = low[rows, :N].double(), low[rows, N:].double(), -torch.exp(a_log.double())
+        S = start[slot].double().view(inner, N).clone()
+        for t in range(m):
+            S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[at + t].double())[:, None] * B[t][None, :]
+            want.append((S @ C[t] + D.double() * x[at + t].double()) * P.silu(z[at + t].double()))
+        ends[slot] = S
+        at += m
+    want = torch.stack(want)
+    dev = lambda t: t.to(DEV)
+    seg_start, seg_len, row_slot, _ = _segs(lens, slots, [0] * len(lens))
+    outs = {}
+    for how in ("chunks", "in a row"):
+        state = dev(start).clone()
+        out = torch.empty(n, inner, device=DEV, dtype=torch.bfloat16)
+        ops.ssm_scan(dev(x), dev(dt_pre), dev(dt_b), dev(low), 0, N, dev(z), dev(a_log), dev(D), seg_start, seg_len, row_slot, state, out, N,
+                     rows_per_request=lens if how == "chunks" else None)
+        outs[how] = out.float().cpu()
+        assert relative_error(out, want) < 4e-3, how
+        for slot, S in ends.items():
+            assert relative_error(state[slot].view(inner, N), S) < 3e-5, (how, slot)
+        assert all(torch.equal(state[s].cpu(), start[s]) for s in range(4) if s not in slots)
+    assert relative_error(outs["chunks"], outs["in a row"].double()) < 2e-3            # (either is one rounding to 8 bits away from the same 32-bit number)
+    assert relative_error(outs["chunks"][:, 0], want[:, 0]) < 4e-3
+
+
 @pytest.mark.parametrize("experts, top", [(5, 2), (16, 1), (3, 3), (64, 8), (130, 4), (1, 1)])
 def test_the_router_s_choice(experts, top):
     from geneinfer_amd.kernels import ops
