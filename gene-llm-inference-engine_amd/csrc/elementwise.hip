@@ -418,7 +418,8 @@ GI_API int gi_rmsnorm_add(const float* y, const void* w, int w_dtype, float* x, 
 // this layer's values (with their bias, before any blending) for such a reader.
 // `flags`: NRS_NEIGHBOURS turns the pairs (2i, 2i + 1), i < rot/2, instead (angle i for pair i); NRS_UNIT_RMS divides every query and
 // key head by its root mean square without weights (q_norm and k_norm must then be absent); NRS_NORM_LAST takes the norm, of
-// either form, behind the rotation instead of in front of it.
+// either form, behind the rotation instead of in front of it.  `v_scale` multiplies the values on their way into the pages (the
+// attention's result is linear in them: a layer that weighs its attention's result can weigh the values instead).
 constexpr int NRS_MAX_HD = 512;
 constexpr int NRS_NEIGHBOURS = 1, NRS_UNIT_RMS = 2, NRS_NORM_LAST = 4;
 
@@ -431,7 +432,8 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
                                                             int page_size, int n_heads, int n_kv, int hd, int vd,
                                                             const float* __restrict__ q_bias, const float* __restrict__ k_bias,
                                                             const float* __restrict__ v_bias, const float* __restrict__ v_other, long ld_other,
-                                                            const float* __restrict__ v_blend, float* __restrict__ v_keep, long ld_keep, int flags) {
+                                                            const float* __restrict__ v_blend, float* __restrict__ v_keep, long ld_keep, int flags,
+                                                            float v_scale) {
     __shared__ float s[NRS_MAX_HD];
     const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
@@ -445,7 +447,7 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
             if (v_bias) x += v_bias[h * vd + d];
             if (v_keep) v_keep[(size_t)t * ld_keep + h * vd + d] = x;
             if (v_other) x = (1.0f - blend) * x + blend * v_other[(size_t)t * ld_other + h * vd + d];
-            store_f32(vbase, (size_t)d * page_size, x);
+            store_f32(vbase, (size_t)d * page_size, v_scale * x);
         }
         return;
     }
@@ -497,7 +499,7 @@ GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, lo
                               const int* table, int table_stride, void* q_out, int q_dtype, void* cache, int cache_dtype, long page_stride,
                               int page_size, int n_rows, int n_heads, int n_kv, int hd, int vd, const float* q_bias, const float* k_bias,
                               const float* v_bias, const float* v_other, long ld_other, const float* v_blend, float* v_keep, long ld_keep,
-                              int flags, hipStream_t stream) {
+                              int flags, float v_scale, hipStream_t stream) {
     GI_REQUIRE(!(flags & NRS_UNIT_RMS) || (q_norm == nullptr && k_norm == nullptr), "norm_rope_store: heads divided by their root mean square have no norm weights");
     GI_REQUIRE(!(flags & NRS_NEIGHBOURS) || rot % 2 == 0, "norm_rope_store: neighbouring pairs need an even number of turned channels");
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && hd > 0 && hd <= NRS_MAX_HD && vd > 0, "norm_rope_store: bad sizes (rows %d heads %d kv %d hd %d vd %d)",
@@ -513,7 +515,7 @@ GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, lo
 #define LAUNCH(TQ, TC, TW)                                                                                                                    \
     norm_rope_store_kernel<TQ, TC, TW><<<grid, 64, 0, stream>>>(q, k, v, ldq, ldk, ldv, (const TW*)q_norm, (const TW*)k_norm, eps, cos_t, sin_t, rot, pos, \
                                                                 slot, table, table_stride, (TQ*)q_out, (TC*)cache, page_stride, page_size, n_heads, n_kv, hd, vd, \
-                                                                q_bias, k_bias, v_bias, v_other, ld_other, v_blend, v_keep, ld_keep, flags)
+                                                                q_bias, k_bias, v_bias, v_other, ld_other, v_blend, v_keep, ld_keep, flags, v_scale)
     if (q_dtype == GI_F32 && cache_dtype == GI_F32 && norm_dtype == GI_F32) LAUNCH(float, float, float);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_F32) LAUNCH(bf16_t, bf16_t, float);

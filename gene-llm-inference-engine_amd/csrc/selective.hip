@@ -131,7 +131,7 @@ __global__ __launch_bounds__(64) void ssm_scan_kernel(const float* __restrict__ 
                                                      const float* __restrict__ a_log, const float* __restrict__ d_skip, const int* __restrict__ seg_start,
                                                      const int* __restrict__ seg_len, const int* __restrict__ row_slot, float* __restrict__ state,
                                                      long state_stride, TO* __restrict__ out, long ldo, int inner, int n_state, int n_segs, int chunk_rows,
-                                                     float* __restrict__ ends, float* __restrict__ sums) {
+                                                     float* __restrict__ ends, float* __restrict__ sums, float out_scale) {
     ScanChunk ch;
     if (PHASE == 0) {
         ch.t0 = seg_start[blockIdx.x], ch.n_rows = seg_len[blockIdx.x], ch.index = 0, ch.last = 1;
@@ -203,7 +203,7 @@ __global__ __launch_bounds__(64) void ssm_scan_kernel(const float* __restrict__ 
             }
             acc += quad_moved<0xB1>(acc);                          // lanes 1 apart: quad_perm [1, 0, 3, 2]
             acc += quad_moved<0x4E>(acc);                          // lanes 2 apart: quad_perm [2, 3, 0, 1]
-            y[j] = fmaf(skip, now.x[j], acc) * now.z[j];
+            y[j] = fmaf(skip, now.x[j], acc) * now.z[j] * out_scale;
         }
         if (PHASE != 1 && live && part == 0) {
 #pragma unroll
@@ -301,7 +301,7 @@ GI_API int gi_ssm_tail(const float* pre, long ld, int n_taps, const int* seg_sta
 GI_API int gi_ssm_scan(const float* x, const float* dt_pre, long ld_dt, const float* dt_bias, const float* bc, long ld_bc, int b_off, int c_off, const float* z,
                        long ld_z, const float* a_log, const float* d_skip, const int* seg_start, const int* seg_len, int n_segs, const int* row_slot,
                        float* state, long state_stride, void* out, int out_dtype, long ldo, int inner, int n_state, int n_chunks, int chunk_rows, float* ends,
-                       float* sums, hipStream_t stream) {
+                       float* sums, float out_scale, hipStream_t stream) {
     GI_REQUIRE(n_segs > 0 && inner > 0 && n_state > 0 && n_state <= 256 && ld_dt >= inner && ld_z >= inner && ldo >= inner && b_off >= 0 && c_off >= 0
                && ld_bc >= b_off + n_state && ld_bc >= c_off + n_state && state_stride >= (long)inner * n_state,
                "ssm_scan: bad sizes (requests %d, channels %d, states %d)", n_segs, inner, n_state);
@@ -313,14 +313,14 @@ GI_API int gi_ssm_scan(const float* x, const float* dt_pre, long ld_dt, const fl
     do {                                                                                                                                                      \
         if (n_chunks == 0) {                                                                                                                                  \
             ssm_scan_kernel<NPL, RB, QUICK, 0, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
-                                                                            seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, 0, nullptr, nullptr); \
+                                                                            seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, 0, nullptr, nullptr, out_scale); \
         } else {                                                                                                                                              \
             dim3 by_chunk(n_chunks, grid.y);                                                                                                                  \
             ssm_scan_kernel<NPL, RB, QUICK, 1, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
-                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums); \
+                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums, out_scale); \
             ssm_carry_kernel<NPL, QUICK><<<grid, 64, 0, stream>>>(a_log, seg_start, seg_len, row_slot, state, state_stride, inner, n_state, chunk_rows, ends, sums); \
             ssm_scan_kernel<NPL, RB, QUICK, 2, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
-                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums); \
+                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums, out_scale); \
         }                                                                                                                                                     \
     } while (0)
 #define BY_STATES(QUICK, TO)                                     \

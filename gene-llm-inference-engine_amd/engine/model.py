@@ -48,6 +48,11 @@ class DecoderModel:
         self.after_embedding = [row_transform_class(t)(t, tensors, dtype, device) for t in spec.after_embedding]
         self.after_head = [row_transform_class(t)(t, tensors, dtype, device) for t in spec.after_head]
         self.run_order = spec.run_order
+        for e in spec.run_order:                   # a mixer whose pages another entry reads keeps nothing but keys and values there
+            if e.cache_of is not None:
+                shared = getattr(getattr(self.layers[spec.run_order[e.cache_of].layer], "mixer", None), "pages_are_shared", None)
+                if shared is not None:
+                    shared()
         # parts that change the residual stream between layers: behind a layer (every time it runs), before a run-order entry
         self.after_layer = [[stream_part_class(t)(t, tensors, dtype, device) for t in l.after] for l in spec.layers]
         self.before_entry = [None if e.before is None else stream_part_class(e.before)(e.before, tensors, dtype, device) for e in spec.run_order]
@@ -100,7 +105,7 @@ class DecoderModel:
                 handed = None
             for part in extras:
                 part.forward(x, ctx)
-            if trace is not None:
+            if extras and trace is not None:
                 trace("layer_out", i, x)
         ctx.trace = None
         if n_logit_rows == 0:
@@ -142,7 +147,7 @@ class DecoderModel:
     def set_trace(self, trace) -> None:
         """Debugging, as the reference's Model::set_trace (src/model/model.h): `trace(tag, run-order entry or -1, rows)` is
         called with the step's residual stream after the embedding ("embedding"), after each half of every block
-        ("attn_out", "ffn_out"), after everything that belongs to a run-order entry ("layer_out") and with the normed rows that the logits are taken from ("final_norm").  While a trace is
+        ("attn_out", "ffn_out"), behind the parts that follow a block, where a layer has such ("layer_out"), and with the normed rows that the logits are taken from ("final_norm").  While a trace is
         set no step is replayed from a captured graph."""
         self.trace = trace
 

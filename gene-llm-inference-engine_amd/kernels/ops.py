@@ -40,7 +40,7 @@ _SIGNATURES = {
     "gi_rmsnorm_add_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_long, c_long, c_long, c_void_p],
     "gi_norm_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int,
                            c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_void_p],
+                           c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_float, c_void_p],
     "gi_concat_rows": [c_void_p, c_long, c_int, c_void_p, c_long, c_int, c_void_p, c_int, c_long, c_int, c_void_p],
     "gi_add_weighted": [c_void_p, c_long, c_void_p, c_long, c_float, c_void_p, c_long, c_float, c_int, c_int, c_void_p],
     "gi_add_vector": [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -48,7 +48,7 @@ _SIGNATURES = {
     "gi_ssm_conv": [c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gi_ssm_tail": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p],
     "gi_ssm_scan": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                    c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+                    c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p],
     "gi_route_top": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_route_rows": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
@@ -510,7 +510,7 @@ def rmsnorm_add_norm(y, weight, eps, x, next_weight, next_eps, out):
 
 
 def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, positions, slots, table, q_out, cache, page_size, n_heads, n_kv, hd, vd,
-                    biases=None, blend=None, keep=None, neighbours=False, unit_rms=False, norm_last=False):
+                    biases=None, blend=None, keep=None, neighbours=False, unit_rms=False, norm_last=False, v_scale=1.0):
     """The general form of `rope_store`: every query and key head is first RMS-normed with q_norm / k_norm [hd] (None: not), then
     the pairs (i, i + rotary_dim/2) of its first rotary_dim channels are turned (cos, sin float32 [n, rotary_dim/2]; None: not);
     queries go to q_out, keys and the values (vd channels a head) into the cache's pages.  k None: the pages are another layer's.
@@ -518,7 +518,8 @@ def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, position
     the values that go into the pages are (1 - weight) v + weight other, other float32 [n, kv_heads*vd] (another layer's values of
     the same rows), weight one float32 number on the device.  keep: float32 [n, kv_heads*vd], gets this layer's values (with
     their bias, before any blending).  neighbours: the pairs turned are (2i, 2i + 1).  unit_rms: every query and key head is divided
-    by its root mean square (eps inside the root), without weights.  norm_last: the heads' norm comes behind the rotation."""
+    by its root mean square (eps inside the root), without weights.  norm_last: the heads' norm comes behind the rotation.
+    v_scale: multiplies the values on their way into the pages."""
     if unit_rms and (q_norm is not None or k_norm is not None):
         raise KernelError("norm_rope_store: heads divided by their root mean square have no norm weights")
     _dev(q, k, v, q_norm, k_norm, cos, sin, positions, slots, table, q_out, cache)
@@ -563,7 +564,7 @@ def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, position
           slots.data_ptr(), _ptr(table) if k is not None else None, table.stride(0) if k is not None else 0, q_out.data_ptr(),
           _code(q_out, "norm_rope_store: q_out"), _ptr(cache) if k is not None else None, cache_code, cache.stride(0) if k is not None else 0,
           int(page_size), n, n_heads, n_kv, hd, vd, _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), _ptr(other), other.stride(0) if other is not None else 0,
-          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, (1 if neighbours else 0) | (2 if unit_rms else 0) | (4 if norm_last else 0), _stream())
+          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, (1 if neighbours else 0) | (2 if unit_rms else 0) | (4 if norm_last else 0), float(v_scale), _stream())
 
 
 def xielu(x, out, params):
@@ -1515,14 +1516,15 @@ SSM_CHUNK_ROWS = 64            # rows of a chunk where a long run of rows is cut
 SSM_CHUNKS_FROM = 128          # rows of a step's longest request from which that is done
 
 
-def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out, n_state, rows_per_request=None):
+def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out, n_state, rows_per_request=None, out_scale=1.0):
     """The recurrence over every request's rows, from its state slot and back into it; out [n, inner] = (read-out + D x) * SiLU(z).
     x float32 [n, inner] contiguous; dt_pre, z float32 [n, inner] (any row stride); low float32 [n, >= offsets + n_state] holds B and
     C of every row at the two offsets; dt_bias, d_skip float32 [inner]; a_log float32 [inner, n_state].
     rows_per_request: the requests' numbers of rows as the host knows them (what seg_len holds).  Given, with results stored as
     bfloat16 and a request of SSM_CHUNKS_FROM rows or more, the rows are cut into chunks of SSM_CHUNK_ROWS that run at once (every
     chunk from a zero state first, then the states the chunks start from, then every chunk with its results): the same sums in
-    another order, so the results differ by 32-bit rounding from those of rows taken one after the other."""
+    another order, so the results differ by 32-bit rounding from those of rows taken one after the other.
+    out_scale multiplies what is stored."""
     _dev(x, dt_pre, dt_bias, low, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out)
     n, inner = x.shape
     _f32_rows(dt_pre, "ssm_scan: the step sizes", n, inner)
@@ -1546,7 +1548,7 @@ def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start,
         sums = torch.empty((n_chunks, inner), dtype=torch.float32, device=x.device)
     _call("gi_ssm_scan", x.data_ptr(), dt_pre.data_ptr(), dt_pre.stride(0), dt_bias.data_ptr(), low.data_ptr(), low.stride(0), int(b_off), int(c_off), z.data_ptr(),
           z.stride(0), a_log.data_ptr(), d_skip.data_ptr(), seg_start.data_ptr(), seg_len.data_ptr(), seg_start.numel(), row_slot.data_ptr(), state.data_ptr(),
-          state.stride(0), out.data_ptr(), _code(out, "ssm_scan: out"), out.stride(0), inner, n_state, n_chunks, SSM_CHUNK_ROWS, _ptr(ends), _ptr(sums), _stream())
+          state.stride(0), out.data_ptr(), _code(out, "ssm_scan: out"), out.stride(0), inner, n_state, n_chunks, SSM_CHUNK_ROWS, _ptr(ends), _ptr(sums), float(out_scale), _stream())
     return out
 
 

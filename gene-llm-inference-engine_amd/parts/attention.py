@@ -213,10 +213,22 @@ class Attention(Mixer):
         ops.norm_rope_store(q, k, v, self.q_norm, self.k_norm if k is not None else None, s.qk_norm_eps, cos, sin, turned, ctx.row_pos, ctx.row_slot,
                             cache.table, q_ready, cache.kv, cache.page_size, s.n_heads, s.n_kv_heads, s.head_dim, vd,
                             biases=biases if any(b is not None for b in biases) else None, blend=blend, keep=keep, neighbours=neighbours,
-                            unit_rms=self.unit_rms, norm_last=self.unit_rms)
+                            unit_rms=self.unit_rms, norm_last=self.unit_rms, v_scale=self.out_scale)
         att = torch.empty((T, s.n_heads * vd), dtype=cache.kv.dtype, device=ctx.device)
         return ops.attention_general(q_ready, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, page_size=cache.page_size,
                                      value_dim=vd, window=s.window, chunk=s.chunk, scale=s.scale, sinks=self.sinks, gate=gate)
+
+    out_scale = 1.0
+
+    def set_out_scale(self, scale: float) -> bool:
+        """Multiplies the mixer's result by `scale`, where that costs nothing: the general path's values are weighed on their way into
+        the layer's own pages (the attention is linear in them).  False: the caller weighs the result itself.  (Another layer that
+        reads these pages would read the weighed values: a layer whose pages are shared is not asked.)"""
+        s = self.spec
+        if not (self.general and s.k_proj is not None and s.value_family is None and s.head_gate is None):
+            return False
+        self.out_scale = float(scale)
+        return True
 
     def input_weight(self):
         """The first product's matrix, for a block that makes several parts' first products in one; None where the plain path's

@@ -29,6 +29,11 @@ class SelectiveScan(Mixer):
     accepts_deferred_norm = True      # its input goes into `linear` only
     hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
     can_overwrite = True
+    out_scale = 1.0                   # multiplies the mixer's result (`set_out_scale`: inside the scan's kernel, before the output product)
+
+    def set_out_scale(self, scale: float) -> bool:
+        self.out_scale = float(scale)
+        return True
 
     def takes_handed_norm(self, n_rows: int) -> bool:
         return self.in_dtype == torch.bfloat16 and takes_handed_norm(self.w_in, n_rows)
@@ -94,7 +99,7 @@ class SelectiveScan(Mixer):
         linear(low[:, :R], self.w_dt, dt_pre)           # (32-bit rows: the step sizes' product keeps them)
         mid = torch.empty((T, inner), dtype=self.mid_dtype, device=dev)
         ops.ssm_scan(x, dt_pre, self.dt_bias, low, R, R + N, z, self.a_log, self.d_skip, seg_start, seg_len, ctx.row_slot, cache.state, mid, N,
-                     rows_per_request=ctx.seg_len)
+                     rows_per_request=ctx.seg_len, out_scale=self.out_scale)
         if overwrite:
             linear(mid, self.w_o, residual)
             return None

@@ -61,15 +61,17 @@ def rotate_neighbours(x, dims, base):
     return out
 
 
-def attention(h, wq, wk, wv, wo, *, heads, kv_heads, dim, vdim, scale, rot_dims, rot_base, eps, store=same):
-    """Causal softmax attention with grouped key/value heads; q and k are turned and then divided by their root mean square."""
+def attention(h, wq, wk, wv, wo, *, heads, kv_heads, dim, vdim, scale, rot_dims, rot_base, eps, store=same, weight=1.0):
+    """Causal softmax attention with grouped key/value heads; q and k are turned and then divided by their root mean square.
+    `weight` multiplies the result; it is taken in on the values (the result is linear in them), which is where an engine that
+    stores them rounded has it."""
     T = h.shape[0]
     q = (h @ wq.T).reshape(T, heads, dim)
     k = (h @ wk.T).reshape(T, kv_heads, dim)
     v = (h @ wv.T).reshape(T, kv_heads, vdim)
     if rot_dims:
         q, k = rotate_neighbours(q, rot_dims, rot_base), rotate_neighbours(k, rot_dims, rot_base)
-    q, k, v = store(rms_norm(q, None, eps)), store(rms_norm(k, None, eps)), store(v)
+    q, k, v = store(rms_norm(q, None, eps)), store(rms_norm(k, None, eps)), store(weight * v)
     per = heads // kv_heads
     out = torch.zeros(T, heads, vdim, dtype=h.dtype)
     seen = torch.tril(torch.ones(T, T, dtype=torch.bool))
@@ -91,8 +93,9 @@ def causal_convolution(x, taps, bias):
     return out + bias
 
 
-def selective_scan(h, w_in, conv, conv_b, w_x, w_dt, dt_b, a_log, d_skip, w_o, *, state, dt_rank, store=same):
-    """S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n;  y_c = S[c, :] . C + D_c x_c;  out = W_o (y * silu(z))."""
+def selective_scan(h, w_in, conv, conv_b, w_x, w_dt, dt_b, a_log, d_skip, w_o, *, state, dt_rank, store=same, weight=1.0):
+    """S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n;  y_c = S[c, :] . C + D_c x_c;  out = W_o (y * silu(z)), times `weight`
+    (taken in before the last product)."""
     T = h.shape[0]
     inner = w_in.shape[0] // 2
     xz = h @ w_in.T
@@ -107,7 +110,7 @@ def selective_scan(h, w_in, conv, conv_b, w_x, w_dt, dt_b, a_log, d_skip, w_o, *
     for t in range(T):
         S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :]
         y[t] = S @ C[t] + d_skip * x[t]
-    return store(y * silu(z)) @ w_o.T
+    return store(weight * y * silu(z)) @ w_o.T
 
 
 # ------------------------------------------------------------------------------------------------------- feed-forwards
@@ -141,10 +144,10 @@ def _mixer(h, cfg, w, p, eps, store):
     left, right = cfg["left"], cfg["right"]
     a = attention(h, w[p + "left.q"], w[p + "left.k"], w[p + "left.v"], w[p + "left.o"], heads=left["heads"], kv_heads=left["kv_heads"],
                   dim=left["dim"], vdim=left["vdim"], scale=left["scale"], rot_dims=left["rot"]["dims"] if left.get("rot") else 0,
-                  rot_base=left["rot"]["base"] if left.get("rot") else 1.0, eps=eps, store=store)
+                  rot_base=left["rot"]["base"] if left.get("rot") else 1.0, eps=eps, store=store, weight=cfg["left_scale"])
     b = selective_scan(h, w[p + "right.in"], w[p + "right.conv"], w[p + "right.conv.b"], w[p + "right.x"], w[p + "right.dt"], w[p + "right.dt.b"],
-                       w[p + "right.A_log"], w[p + "right.D"], w[p + "right.o"], state=right["state"], dt_rank=right["dt_rank"], store=store)
-    return cfg["left_scale"] * a + cfg["right_scale"] * b
+                       w[p + "right.A_log"], w[p + "right.D"], w[p + "right.o"], state=right["state"], dt_rank=right["dt_rank"], store=store, weight=cfg["right_scale"])
+    return a + b
 
 
 def _feed_forward(h, cfg, w, p, store):

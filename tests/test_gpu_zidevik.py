@@ -395,12 +395,13 @@ def test_the_residual_stream_after_every_layer_run(folders, name):
     P.forward(cfg, stored_weights(folders[name]), tokens, streams=want)
     runner = make_runner(folders, name, "float32")
     runner.open("r")
-    got = []
-    runner.model.set_trace(lambda tag, i, rows: got.append(rows.float().cpu()) if tag == "layer_out" else None)
+    last = {}                                      # per run-order entry, the stream as the entry leaves it: behind the block, or behind what follows it
+    runner.model.set_trace(lambda tag, i, rows: last.__setitem__(i, rows.float().cpu()) if tag in ("ffn_out", "layer_out") else None)
     try:
         feed(runner, "r", tokens, [len(tokens)])
     finally:
         runner.model.set_trace(None)
+    got = [last[i] for i in sorted(last)]
     assert len(got) == len(want) == len(P.run_order(cfg))
     for i, (g, w) in enumerate(zip(got, want)):
         assert relative_error(g, w) < 2e-5, f"{name}: the stream differs behind layer run {i} (layer {P.run_order(cfg)[i][0]})"
