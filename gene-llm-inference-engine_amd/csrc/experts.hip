@@ -142,8 +142,18 @@ __global__ __launch_bounds__(256) void route_rows_kernel(const TA* __restrict__ 
     const TA* a = h + t * ldh;
     for (int e = wave; e < n_experts; e += 4) {
         const TW* w = router + (size_t)e * ldr;
+        // a lane takes eight neighbouring columns at a time, four such pieces asked for at once; the columns left over one by one
         float s = 0.f;
-        for (int d = lane; d < width; d += 64) s = fmaf(load_f32(w, d), load_f32(a, d), s);
+        const int whole = width & ~7;
+#pragma unroll 4
+        for (int d = lane * 8; d < whole; d += 512) {
+            float wv[8], av[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) wv[i] = load_f32(w, d + i), av[i] = load_f32(a, d + i);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s = fmaf(wv[i], av[i], s);
+        }
+        for (int d = whole + lane; d < width; d += 64) s = fmaf(load_f32(w, d), load_f32(a, d), s);
         s = wave_sum(s);
         if (lane == 0) {
             zs[e] = s;
