@@ -701,6 +701,53 @@ __global__ __launch_bounds__(64) void gate_token_columns_kernel(const float* __r
     }
 }
 
+// The same behind a product of a few rows, all in one: out[t, j] = act(W[j] . a[t]) * table[tokens[t], first + j] with a[t] the 32-bit row
+// x[t] as a product reads it (rounded to bfloat16 where `round_rows`).  One wave per (row, output): a lane takes eight neighbouring
+// columns at a time, the lanes' sums are added by a butterfly.
+template <typename TW, typename TT, typename TO>
+__global__ __launch_bounds__(256) void gate_token_columns_rows_kernel(const float* __restrict__ x, long ldx, const TW* __restrict__ w, long ldw, int width,
+                                                                     const TT* __restrict__ table, long ldt, int first, const int* __restrict__ tokens,
+                                                                     TO* __restrict__ out, long ldo, int dim, int act, int round_rows) {
+    const size_t t = blockIdx.x;
+    const int j = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (j >= dim) return;
+    const float* a = x + t * ldx;
+    const TW* wj = w + (size_t)j * ldw;
+    float s = 0.f;
+    const int whole = width & ~7;
+#pragma unroll 4
+    for (int d = lane * 8; d < whole; d += 512) {
+        float wv[8], av[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) wv[i] = load_f32(wj, d + i), av[i] = a[d + i];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) s = fmaf(wv[i], round_rows ? bf16_to_f32(f32_to_bf16(av[i])) : av[i], s);
+    }
+    for (int d = whole + lane; d < width; d += 64) s = fmaf(load_f32(wj, d), round_rows ? bf16_to_f32(f32_to_bf16(a[d])) : a[d], s);
+    s = wave_sum(s);
+    if (lane == 0) {
+        const float g = act == 1 ? 0.5f * s * (1.0f + tanhf(0.7978845608028654f * (s + 0.044715f * s * s * s))) : s / (1.0f + expf(-s));
+        store_f32(out + t * ldo, j, g * load_f32(table + (size_t)tokens[t] * ldt + first, j));
+    }
+}
+
+GI_API int gi_gate_token_columns_rows(const float* x, long ldx, const void* w, int w_dtype, long ldw, int width, const void* table, int table_dtype, long ldt, int first,
+                                      const int* tokens, void* out, int out_dtype, long ldo, int n_rows, int dim, int act, int round_rows, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && dim > 0 && width > 0 && ldx >= width && ldw >= width && ldo >= dim && first >= 0 && ldt >= first + dim && (act == 0 || act == 1),
+               "gate_token_columns_rows: bad sizes (rows %d, width %d, dim %d, columns from %d of %ld)", n_rows, width, dim, first, ldt);
+    dim3 grid(n_rows, (dim + 3) / 4);
+    GI_REQUIRE(grid.y <= 65535, "gate_token_columns_rows: too many columns");
+#define LAUNCH(TW, TT, TO)                                                                                                                            \
+    gate_token_columns_rows_kernel<TW, TT, TO><<<grid, 256, 0, stream>>>(x, ldx, (const TW*)w, ldw, width, (const TT*)table, ldt, first, tokens, (TO*)out, ldo, dim, act, \
+                                                                         round_rows)
+    if (w_dtype == GI_BF16 && table_dtype == GI_BF16 && out_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
+    else if (w_dtype == GI_F32 && table_dtype == GI_F32 && out_dtype == GI_F32) LAUNCH(float, float, float);
+    else return gi_fail("gate_token_columns_rows: dtypes (%d, %d, %d) are not served", w_dtype, table_dtype, out_dtype);
+#undef LAUNCH
+    GI_CHECK_LAUNCH("gate_token_columns_rows");
+    return 0;
+}
+
 GI_API int gi_gate_token_columns(const float* u, long ldu, const void* table, int table_dtype, long ldt, int first, const int* tokens, void* out, int out_dtype,
                                  long ldo, int n_rows, int dim, int act, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && dim > 0 && ldu >= dim && ldo >= dim && first >= 0 && ldt >= first + dim && (act == 0 || act == 1),

@@ -16,7 +16,7 @@
 
 namespace {
 
-constexpr int SSM_MAX_TAPS = 8;
+constexpr int SSM_MAX_TAPS = 16;
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
@@ -125,13 +125,17 @@ __device__ __forceinline__ bool find_chunk(ScanChunk& ch, int g, const int* __re
     return false;
 }
 
-template <int NPL, int RB, bool QUICK, int PHASE, typename TO>
+// Steps of single rows take the kernel with RB = 1 (`single_rows`: the host says so; more rows would be right too, only slow).
+// FUSED_DT (such steps): the step sizes' product is made here, dt_pre[t, c] = w_dt[c] . low[t, dt_off .. dt_off + dt_rank),
+// a channel's four lanes a quarter of the sum each; `dt_pre` is then not read.
+template <int NPL, int RB, bool QUICK, int PHASE, bool FUSED_DT, typename TO>
 __global__ __launch_bounds__(64) void ssm_scan_kernel(const float* __restrict__ x, const float* __restrict__ dt_pre, long ld_dt, const float* __restrict__ dt_bias,
                                                      const float* __restrict__ bc, long ld_bc, int b_off, int c_off, const float* __restrict__ z, long ld_z,
                                                      const float* __restrict__ a_log, const float* __restrict__ d_skip, const int* __restrict__ seg_start,
                                                      const int* __restrict__ seg_len, const int* __restrict__ row_slot, float* __restrict__ state,
                                                      long state_stride, TO* __restrict__ out, long ldo, int inner, int n_state, int n_segs, int chunk_rows,
-                                                     float* __restrict__ ends, float* __restrict__ sums, float out_scale) {
+                                                     float* __restrict__ ends, float* __restrict__ sums, float out_scale,
+                                                     const bf16_t* __restrict__ w_dt, long ld_w, int dt_off, int dt_rank, int dt_vec) {
     ScanChunk ch;
     if (PHASE == 0) {
         ch.t0 = seg_start[blockIdx.x], ch.n_rows = seg_len[blockIdx.x], ch.index = 0, ch.last = 1;
@@ -162,7 +166,33 @@ __global__ __launch_bounds__(64) void ssm_scan_kernel(const float* __restrict__ 
         for (int j = 0; j < RB; ++j) {
             const size_t t = t0 + min(r0 + j, n_rows - 1);          // (rows behind the last ask for the last again)
             rows.x[j] = x[t * inner + cc];
-            rows.dt[j] = dt_pre[t * ld_dt + cc];
+            if (FUSED_DT && r0 + j >= n_rows) {
+                rows.dt[j] = 0.f;                                 // (a row behind the last: nothing of it is kept)
+            } else if (FUSED_DT) {
+                // a lane takes one run of neighbouring columns: in pieces of eight where the rank and the rows' places allow (dt_vec)
+                const int per = (dt_rank + 3) / 4, r_lo = min(part * per, dt_rank), r_hi = min(r_lo + per, dt_rank);
+                const float* lo = bc + t * ld_bc + dt_off;
+                const bf16_t* wr = w_dt + (size_t)cc * ld_w;
+                float s = 0.f;
+                int r = r_lo;
+                if (dt_vec) {
+#pragma unroll 4
+                    for (; r + 8 <= r_hi; r += 8) {
+                        const uint4 w8 = *reinterpret_cast<const uint4*>(wr + r);
+                        const float4 a = *reinterpret_cast<const float4*>(lo + r), b = *reinterpret_cast<const float4*>(lo + r + 4);
+                        s = fmaf(a.x, __uint_as_float(w8.x << 16), s), s = fmaf(a.y, __uint_as_float(w8.x & 0xffff0000u), s);
+                        s = fmaf(a.z, __uint_as_float(w8.y << 16), s), s = fmaf(a.w, __uint_as_float(w8.y & 0xffff0000u), s);
+                        s = fmaf(b.x, __uint_as_float(w8.z << 16), s), s = fmaf(b.y, __uint_as_float(w8.z & 0xffff0000u), s);
+                        s = fmaf(b.z, __uint_as_float(w8.w << 16), s), s = fmaf(b.w, __uint_as_float(w8.w & 0xffff0000u), s);
+                    }
+                }
+                for (; r < r_hi; ++r) s = fmaf(lo[r], bf16_to_f32(wr[r]), s);
+                s += quad_moved<0xB1>(s);
+                s += quad_moved<0x4E>(s);
+                rows.dt[j] = s;
+            } else {
+                rows.dt[j] = dt_pre[t * ld_dt + cc];
+            }
             if (PHASE != 1) rows.z[j] = z[t * ld_z + cc];
 #pragma unroll
             for (int i = 0; i < NPL; ++i) {
@@ -301,26 +331,41 @@ GI_API int gi_ssm_tail(const float* pre, long ld, int n_taps, const int* seg_sta
 GI_API int gi_ssm_scan(const float* x, const float* dt_pre, long ld_dt, const float* dt_bias, const float* bc, long ld_bc, int b_off, int c_off, const float* z,
                        long ld_z, const float* a_log, const float* d_skip, const int* seg_start, const int* seg_len, int n_segs, const int* row_slot,
                        float* state, long state_stride, void* out, int out_dtype, long ldo, int inner, int n_state, int n_chunks, int chunk_rows, float* ends,
-                       float* sums, float out_scale, hipStream_t stream) {
-    GI_REQUIRE(n_segs > 0 && inner > 0 && n_state > 0 && n_state <= 256 && ld_dt >= inner && ld_z >= inner && ldo >= inner && b_off >= 0 && c_off >= 0
+                       float* sums, float out_scale, const void* w_dt, long ld_w, int dt_off, int dt_rank, int single_rows, hipStream_t stream) {
+    GI_REQUIRE(n_segs > 0 && inner > 0 && n_state > 0 && n_state <= 256 && (dt_pre == nullptr || ld_dt >= inner) && ld_z >= inner && ldo >= inner && b_off >= 0 && c_off >= 0
                && ld_bc >= b_off + n_state && ld_bc >= c_off + n_state && state_stride >= (long)inner * n_state,
                "ssm_scan: bad sizes (requests %d, channels %d, states %d)", n_segs, inner, n_state);
     dim3 grid(n_segs, (inner + 15) / 16);
     GI_REQUIRE(grid.y <= 65535, "ssm_scan: too many channels");
+    // pieces of eight columns of the step sizes' matrix: every lane's run starts at a multiple of eight, in rows that start at multiples of 16 bytes
+    const int dt_vec = w_dt != nullptr && ((dt_rank + 3) / 4) % 8 == 0 && ld_w % 8 == 0 && ((uintptr_t)w_dt & 15) == 0 && ld_bc % 4 == 0 && dt_off % 4 == 0
+                       && ((uintptr_t)bc & 15) == 0;
+    GI_REQUIRE(w_dt == nullptr || (out_dtype == GI_BF16 && n_chunks == 0 && single_rows && dt_rank > 0 && ld_w >= dt_rank && dt_off >= 0 && ld_bc >= dt_off + dt_rank),
+               "ssm_scan: the step sizes' product inside the scan needs bfloat16 results, rows not in chunks, and its columns within the rows of B and C");
+    GI_REQUIRE(w_dt != nullptr || dt_pre != nullptr, "ssm_scan: step sizes, or the matrix that makes them, are needed");
     GI_REQUIRE(n_chunks == 0 || (n_chunks > 0 && chunk_rows > 0 && ends != nullptr && sums != nullptr && out_dtype == GI_BF16),
                "ssm_scan: rows in chunks need the chunks' scratch memory and results stored as bfloat16");
 #define LAUNCH(NPL, RB, QUICK, TO)                                                                                                                            \
     do {                                                                                                                                                      \
-        if (n_chunks == 0) {                                                                                                                                  \
-            ssm_scan_kernel<NPL, RB, QUICK, 0, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
-                                                                            seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, 0, nullptr, nullptr, out_scale); \
+        if (n_chunks == 0 && single_rows && !(QUICK && w_dt != nullptr)) {                                                                                    \
+            ssm_scan_kernel<NPL, 1, QUICK, 0, false, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+                                                                                  seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, 0, nullptr, nullptr, out_scale, \
+                                                                                  nullptr, 0, 0, 0, 0);                                                        \
+        } else if (n_chunks == 0 && QUICK && w_dt != nullptr) {                                                                                               \
+            ssm_scan_kernel<NPL, 1, QUICK, 0, QUICK, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+                                                                                   seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, 0, nullptr, nullptr, out_scale, \
+                                                                                   (const bf16_t*)w_dt, ld_w, dt_off, dt_rank, dt_vec);                                \
+        } else if (n_chunks == 0) {                                                                                                                           \
+            ssm_scan_kernel<NPL, RB, QUICK, 0, false, TO><<<grid, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+                                                                                   seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, 0, nullptr, nullptr, out_scale, \
+                                                                                   nullptr, 0, 0, 0, 0);                                                        \
         } else {                                                                                                                                              \
             dim3 by_chunk(n_chunks, grid.y);                                                                                                                  \
-            ssm_scan_kernel<NPL, RB, QUICK, 1, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
-                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums, out_scale); \
+            ssm_scan_kernel<NPL, RB, QUICK, 1, false, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums, out_scale, nullptr, 0, 0, 0, 0); \
             ssm_carry_kernel<NPL, QUICK><<<grid, 64, 0, stream>>>(a_log, seg_start, seg_len, row_slot, state, state_stride, inner, n_state, chunk_rows, ends, sums); \
-            ssm_scan_kernel<NPL, RB, QUICK, 2, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
-                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums, out_scale); \
+            ssm_scan_kernel<NPL, RB, QUICK, 2, false, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+                                                                                seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums, out_scale, nullptr, 0, 0, 0, 0); \
         }                                                                                                                                                     \
     } while (0)
 #define BY_STATES(QUICK, TO)                                     \

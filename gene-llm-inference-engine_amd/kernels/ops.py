@@ -45,10 +45,12 @@ _SIGNATURES = {
     "gi_add_weighted": [c_void_p, c_long, c_void_p, c_long, c_float, c_void_p, c_long, c_float, c_int, c_int, c_void_p],
     "gi_add_vector": [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
     "gi_gate_token_columns": [c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_void_p],
+    "gi_gate_token_columns_rows": [c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_void_p, c_int, c_long, c_int, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int,
+                                   c_void_p],
     "gi_ssm_conv": [c_void_p, c_long, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gi_ssm_tail": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p],
     "gi_ssm_scan": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                    c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p],
+                    c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
     "gi_route_top": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_route_rows": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
@@ -1468,8 +1470,27 @@ def gate_token_columns(u, table, first, tokens, out, activation="gelu_tanh"):
     return out
 
 
+def gate_token_columns_rows(x, w, table, first, tokens, out, activation="gelu_tanh"):
+    """out[t, j] = act(w[j] . x[t]) * table[tokens[t], first + j] in one launch, for a few rows: x float32 [n, width], read as a product
+    reads rows (rounded to bfloat16 where w is bfloat16); w [dim, width]; out [n, dim] of w's dtype."""
+    _dev(x, w, table, tokens, out)
+    n, width = x.shape
+    dim = w.shape[0]
+    _f32_rows(x, "gate_token_columns_rows: x")
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"gate_token_columns_rows: unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
+    if not (w.shape == (dim, width) and w.stride(1) == 1 and table.dim() == 2 and table.stride(1) == 1 and 0 <= first and first + dim <= table.shape[1]
+            and out.shape == (n, dim) and out.stride(1) == 1 and w.dtype == table.dtype == out.dtype):
+        raise KernelError("gate_token_columns_rows: w [dim, width], a table that holds the columns asked for and out [n, dim], all of one dtype, are needed")
+    _i32(tokens, "gate_token_columns_rows: tokens", n)
+    _call("gi_gate_token_columns_rows", x.data_ptr(), x.stride(0), w.data_ptr(), _code(w, "gate_token_columns_rows: w"), w.stride(0), width, table.data_ptr(),
+          _code(table, "gate_token_columns_rows: table"), table.stride(0), int(first), tokens.data_ptr(), out.data_ptr(), _code(out, "gate_token_columns_rows: out"),
+          out.stride(0), n, dim, ACTIVATIONS[activation], 1 if w.dtype == torch.bfloat16 else 0, _stream())
+    return out
+
+
 # ------------------------------------------------------------------------------------------------------------ the selective scan
-SSM_MAX_TAPS, SSM_MAX_STATES = 8, 256
+SSM_MAX_TAPS, SSM_MAX_STATES = 16, 256
 
 
 def ssm_state_floats(inner, n_state, n_taps) -> int:
@@ -1516,7 +1537,7 @@ SSM_CHUNK_ROWS = 64            # rows of a chunk where a long run of rows is cut
 SSM_CHUNKS_FROM = 128          # rows of a step's longest request from which that is done
 
 
-def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out, n_state, rows_per_request=None, out_scale=1.0):
+def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out, n_state, rows_per_request=None, out_scale=1.0, dt_proj=None):
     """The recurrence over every request's rows, from its state slot and back into it; out [n, inner] = (read-out + D x) * SiLU(z).
     x float32 [n, inner] contiguous; dt_pre, z float32 [n, inner] (any row stride); low float32 [n, >= offsets + n_state] holds B and
     C of every row at the two offsets; dt_bias, d_skip float32 [inner]; a_log float32 [inner, n_state].
@@ -1524,10 +1545,23 @@ def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start,
     bfloat16 and a request of SSM_CHUNKS_FROM rows or more, the rows are cut into chunks of SSM_CHUNK_ROWS that run at once (every
     chunk from a zero state first, then the states the chunks start from, then every chunk with its results): the same sums in
     another order, so the results differ by 32-bit rounding from those of rows taken one after the other.
-    out_scale multiplies what is stored."""
+    out_scale multiplies what is stored.
+    dt_proj = (w_dt, offset) with dt_pre None: the kernel makes the step sizes' product itself, dt_pre = low[:, offset : offset + rank] @
+    w_dt.T, w_dt bfloat16 [inner, rank]; for steps of a few rows whose results are stored as bfloat16."""
     _dev(x, dt_pre, dt_bias, low, z, a_log, d_skip, seg_start, seg_len, row_slot, state, out)
     n, inner = x.shape
-    _f32_rows(dt_pre, "ssm_scan: the step sizes", n, inner)
+    w_dt, dt_off = dt_proj if dt_proj is not None else (None, 0)
+    if (dt_pre is None) == (w_dt is None):
+        raise KernelError("ssm_scan: either the step sizes or the matrix that makes them")
+    if w_dt is not None:
+        _dev(w_dt)
+        if not (w_dt.dtype == torch.bfloat16 and w_dt.dim() == 2 and w_dt.shape[0] == inner and w_dt.stride(1) == 1 and out.dtype == torch.bfloat16
+                and 0 <= dt_off and dt_off + w_dt.shape[1] <= low.shape[1]):
+            raise KernelError("ssm_scan: the step sizes' matrix must be bfloat16 [inner, rank], its columns within `low`, the results bfloat16")
+        if rows_per_request is None or max(rows_per_request) != 1:
+            raise KernelError("ssm_scan: the step sizes' product inside the kernel is for steps of single rows (rows_per_request says so)")
+    else:
+        _f32_rows(dt_pre, "ssm_scan: the step sizes", n, inner)
     _f32_rows(z, "ssm_scan: the gate", n, inner)
     _f32_rows(low, "ssm_scan: B and C", n)
     if not (x.dtype == torch.float32 and x.is_contiguous() and out.shape == (n, inner) and out.stride(1) == 1):
@@ -1540,15 +1574,17 @@ def ssm_scan(x, dt_pre, dt_bias, low, b_off, c_off, z, a_log, d_skip, seg_start,
     _ssm_state(state, inner, n_state, 1, "ssm_scan")
     _i32(row_slot, "ssm_scan: slots", n)
     n_chunks, ends, sums = 0, None, None
-    if rows_per_request is not None and out.dtype == torch.bfloat16 and max(rows_per_request) >= SSM_CHUNKS_FROM:
+    if rows_per_request is not None and out.dtype == torch.bfloat16 and max(rows_per_request) >= SSM_CHUNKS_FROM and w_dt is None:
         if len(rows_per_request) != seg_start.numel() or sum(rows_per_request) != n:
             raise KernelError("ssm_scan: the requests' numbers of rows do not add up to the step's rows")
         n_chunks = sum(-(-int(r) // SSM_CHUNK_ROWS) for r in rows_per_request)
         ends = torch.empty((n_chunks, inner, n_state), dtype=torch.float32, device=x.device)
         sums = torch.empty((n_chunks, inner), dtype=torch.float32, device=x.device)
-    _call("gi_ssm_scan", x.data_ptr(), dt_pre.data_ptr(), dt_pre.stride(0), dt_bias.data_ptr(), low.data_ptr(), low.stride(0), int(b_off), int(c_off), z.data_ptr(),
+    _call("gi_ssm_scan", x.data_ptr(), _ptr(dt_pre), dt_pre.stride(0) if dt_pre is not None else 0, dt_bias.data_ptr(), low.data_ptr(), low.stride(0), int(b_off), int(c_off), z.data_ptr(),
           z.stride(0), a_log.data_ptr(), d_skip.data_ptr(), seg_start.data_ptr(), seg_len.data_ptr(), seg_start.numel(), row_slot.data_ptr(), state.data_ptr(),
-          state.stride(0), out.data_ptr(), _code(out, "ssm_scan: out"), out.stride(0), inner, n_state, n_chunks, SSM_CHUNK_ROWS, _ptr(ends), _ptr(sums), float(out_scale), _stream())
+          state.stride(0), out.data_ptr(), _code(out, "ssm_scan: out"), out.stride(0), inner, n_state, n_chunks, SSM_CHUNK_ROWS, _ptr(ends), _ptr(sums), float(out_scale),
+          _ptr(w_dt), w_dt.stride(0) if w_dt is not None else 0, int(dt_off), w_dt.shape[1] if w_dt is not None else 0,
+          1 if rows_per_request is not None and max(rows_per_request) == 1 else 0, _stream())
     return out
 
 

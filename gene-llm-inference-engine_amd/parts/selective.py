@@ -3,7 +3,7 @@
 One product gives the 32-bit [x | z] of a step's rows.  One kernel takes x through its short convolution (a request's rows
 before this step come from its state) and SiLU; one keeps every request's last rows for the next step's convolution (in a step
 of single rows the kernel before it does that on its way).  A second product makes [dt | B | C] of the convolved rows, a third
-the channels' step sizes from dt.  One kernel steps the states over every request's rows, in order, from the request's state
+the channels' step sizes from dt (in bfloat16 steps of single rows the scan's kernel makes that one on its way).  One kernel steps the states over every request's rows, in order, from the request's state
 slot and back into it, and stores (read-out + D x) * SiLU(z) as the output product reads it.  The step sizes (from the third
 product on: bias, softplus), the decays and their exponentials, B, C, the state and the read-out are 32-bit, whatever the
 compute dtype.  In bfloat16 a request's long run of rows (a prompt) is cut into chunks that run at once (`ops.ssm_scan`); in
@@ -95,11 +95,15 @@ class SelectiveScan(Mixer):
             ops.ssm_tail(pre, s.conv_taps, seg_start, seg_len, ctx.row_slot, cache.state, inner, N)
         low = torch.empty((T, self.w_x.shape[0]), dtype=torch.float32, device=dev)
         linear(x_low, self.w_x, low)
-        dt_pre = torch.empty((T, inner), dtype=torch.float32, device=dev)
-        linear(low[:, :R], self.w_dt, dt_pre)           # (32-bit rows: the step sizes' product keeps them)
         mid = torch.empty((T, inner), dtype=self.mid_dtype, device=dev)
+        dt_pre = dt_proj = None
+        if single_rows and self.mid_dtype == torch.bfloat16 and self.w_dt.dtype == torch.bfloat16:
+            dt_proj = (self.w_dt, 0)                    # (a step of single rows: the scan's kernel makes the step sizes' product on its way)
+        else:
+            dt_pre = torch.empty((T, inner), dtype=torch.float32, device=dev)
+            linear(low[:, :R], self.w_dt, dt_pre)       # (32-bit rows: the step sizes' product keeps them)
         ops.ssm_scan(x, dt_pre, self.dt_bias, low, R, R + N, z, self.a_log, self.d_skip, seg_start, seg_len, ctx.row_slot, cache.state, mid, N,
-                     rows_per_request=ctx.seg_len, out_scale=self.out_scale)
+                     rows_per_request=ctx.seg_len, out_scale=self.out_scale, dt_proj=dt_proj)
         if overwrite:
             linear(mid, self.w_o, residual)
             return None

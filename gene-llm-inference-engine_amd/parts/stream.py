@@ -38,8 +38,17 @@ class TokenSideInput(StreamPart):
     def weights_read_per_step(self):
         return [self.w_gate, self.w_out, self.norm]
 
+    FEW_ROWS = 16      # up to so many rows (bfloat16) the stream's rounding, the first product and the gate are one kernel
+
     def forward(self, x, ctx):
         s, T, dev = self.spec, ctx.n_rows, ctx.device
+        if (T <= self.FEW_ROWS and self.in_dtype == torch.bfloat16 and self.w_gate.dtype == self.table.dtype == self.mid_dtype == torch.bfloat16):
+            g = torch.empty((T, s.dim), dtype=torch.bfloat16, device=dev)
+            ops.gate_token_columns_rows(x, self.w_gate, self.table, s.first_column, ctx.tokens, g, s.activation)
+            y = torch.empty((T, s.hidden_size), dtype=torch.float32, device=dev)
+            linear(g, self.w_out, y)
+            self.norm.add_onto(y, x)
+            return
         rows = x if self.in_dtype == torch.float32 else ops.concat_rows(x, None, torch.empty((T, s.hidden_size), dtype=self.in_dtype, device=dev))
         u = torch.empty((T, s.dim), dtype=torch.float32, device=dev)
         linear(rows, self.w_gate, u)

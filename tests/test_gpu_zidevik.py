@@ -88,7 +88,7 @@ def _segs(seg_lens, slots, pos0):
     return i32(starts), i32(seg_lens), row_slot, row_pos
 
 
-@pytest.mark.parametrize("inner, N, taps", [(40, 5, 3), (72, 17, 4), (30, 1, 1), (17, 33, 3), (9, 2, 8), (256, 16, 4), (64, 100, 2), (20, 130, 5)])
+@pytest.mark.parametrize("inner, N, taps", [(40, 5, 3), (72, 17, 4), (30, 1, 1), (17, 33, 3), (9, 2, 8), (256, 16, 4), (64, 100, 2), (20, 130, 5), (24, 7, 13)])
 def test_selective_scan_kernels(inner, N, taps):
     """Two requests of unequal length in one step; then the longer one again from a fresh slot in steps down to one and two rows:
     the states and the convolutions' tails carry, and the bits do not change.  One channel barely decays, so that what the first
@@ -129,7 +129,8 @@ def test_selective_scan_kernels(inner, N, taps):
         ops.ssm_conv(p, d_taps, d_cb, row_slot, row_pos, state, x, None, N, move_tail=single)
         if not single:
             ops.ssm_tail(p, taps, seg_start, seg_len, row_slot, state, inner, N)
-        ops.ssm_scan(x, dev(dt_pre[rows]), d_db, dev(low[rows]), 2, 2 + N, dev(z[rows]), d_al, d_D, seg_start, seg_len, row_slot, state, out, N)
+        ops.ssm_scan(x, dev(dt_pre[rows]), d_db, dev(low[rows]), 2, 2 + N, dev(z[rows]), d_al, d_D, seg_start, seg_len, row_slot, state, out, N,
+                     rows_per_request=seg_lens)
         return x.cpu(), out.cpu()
 
     x, y = run(slice(0, n), lens, [2, 0], [0, 0])
@@ -158,6 +159,20 @@ def test_selective_scan_kernels(inner, N, taps):
     half = torch.empty(lens[0], inner, device=DEV, dtype=torch.bfloat16)
     ops.ssm_scan(dev(x1.float()), dev(dt_pre[first]), d_db, dev(low[first]), 2, 2 + N, dev(z[first]), d_al, d_D, seg_start, seg_len, row_slot, state, half, N)
     assert relative_error(half, y1) < 4e-3 and relative_error(state[1, :inner * N].view(inner, N), S1) < 3e-5
+    # steps of single rows: the step sizes' product inside the scan's kernel against the same product made in front of it
+    seg_start, seg_len, row_slot, _ = _segs([1, 1, 1], [2, 0, 4], [0, 0, 0])
+    rows3 = slice(0, 3)
+    for R in (7, 64, 96):             # (a rank the lanes take one by one, and ranks they take in pieces of eight)
+        w_dt, low_dt = (0.3 * torch.randn(inner, R, generator=g)).to(torch.bfloat16), torch.randn(3, -(-(R + 2 * N) // 4) * 4, generator=g)
+        made = (low_dt[:, :R].double() @ w_dt.double().T).float()
+        results = []
+        for dt_pre, dt_proj in ((dev(made), None), (None, (dev(w_dt), 0))):
+            state[:] = 0.25
+            out3 = torch.empty(3, inner, device=DEV, dtype=torch.bfloat16)
+            ops.ssm_scan(dev(x1.float()[rows3]), dt_pre, d_db, dev(low_dt), R, R + N, dev(z[rows3]), d_al, d_D, seg_start, seg_len, row_slot, state, out3, N, dt_proj=dt_proj,
+                         rows_per_request=[1, 1, 1])
+            results.append((out3.float().cpu(), state[:, :inner * N].cpu().clone()))
+        assert relative_error(results[1][0], results[0][0].double()) < 4e-3 and relative_error(results[1][1], results[0][1].double()) < 1e-5
     low_copy = torch.empty(5, inner, device=DEV, dtype=torch.bfloat16)
     seg_start, seg_len, row_slot, row_pos = _segs([5], [1], [0])
     state[1] = 0
@@ -373,6 +388,15 @@ def test_rows_side_by_side_weighted_sums_vectors_and_gated_token_columns():
             assert relative_error(out, fn(u.double()) * table.double()[tokens.long()][:, first:first + 6]) < 1e-6
     with pytest.raises(ops.KernelError):
         ops.gate_token_columns(u.to(DEV), table.to(DEV), 45, tokens.to(DEV), out)
+    # a few rows: the product in front of the gate in the same kernel, the rows rounded as a bfloat16 product reads them
+    for width in (37, 300, 1024):
+        rows, w = torch.randn(9, width, generator=g), 0.1 * torch.randn(6, width, generator=g)
+        for dtype, tol in ((torch.float32, 1e-6), (torch.bfloat16, 6e-3)):
+            read = rows.to(dtype).double()
+            want = P.gelu_tanh(read @ w.to(dtype).double().T) * table.to(dtype).double()[tokens.long()][:, 12:18]
+            out = torch.empty(9, 6, device=DEV, dtype=dtype)
+            ops.gate_token_columns_rows(rows.to(DEV), w.to(DEV, dtype), table.to(DEV, dtype), 12, tokens.to(DEV), out)
+            assert relative_error(out, want) < tol
 
 
 # =============================================================================================== whole models
