@@ -361,10 +361,10 @@ GI_API int gi_ssm_scan(const float* x, const float* dt_pre, long ld_dt, const fl
                                                                                    nullptr, 0, 0, 0, 0);                                                        \
         } else {                                                                                                                                              \
             dim3 by_chunk(n_chunks, grid.y);                                                                                                                  \
-            ssm_scan_kernel<NPL, RB, QUICK, 1, false, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+            ssm_scan_kernel<NPL, (RB > 3 ? RB / 4 : 1), QUICK, 1, false, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
                                                                                 seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums, out_scale, nullptr, 0, 0, 0, 0); \
             ssm_carry_kernel<NPL, QUICK><<<grid, 64, 0, stream>>>(a_log, seg_start, seg_len, row_slot, state, state_stride, inner, n_state, chunk_rows, ends, sums); \
-            ssm_scan_kernel<NPL, RB, QUICK, 2, false, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
+            ssm_scan_kernel<NPL, (RB > 3 ? RB / 4 : 1), QUICK, 2, false, TO><<<by_chunk, 64, 0, stream>>>(x, dt_pre, ld_dt, dt_bias, bc, ld_bc, b_off, c_off, z, ld_z, a_log, d_skip, seg_start, \
                                                                                 seg_len, row_slot, state, state_stride, (TO*)out, ldo, inner, n_state, n_segs, chunk_rows, ends, sums, out_scale, nullptr, 0, 0, 0, 0); \
         }                                                                                                                                                     \
     } while (0)
