@@ -71,10 +71,13 @@ class InterleavedRotarySpec:
 
 @dataclass(frozen=True)
 class RmsNormSpec:
+    """x / sqrt(mean(x^2) + eps) * (weight + weight_offset): an architecture that stores its norm weights around zero says
+    weight_offset = 1."""
     kind: ClassVar[str] = "rmsnorm"
     size: int
     eps: float
     weight: str                      # tensor name
+    weight_offset: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -112,6 +115,10 @@ class AttentionSpec:
     # Every query and key head divided by its root mean square over the head (eps `qk_norm_eps` inside the root), without weights and
     # behind the rotation (q_norm and k_norm must then be absent).
     qk_unit_rms: bool = False
+    # q_norm and k_norm taken over all heads of the projection at once (tensors [heads*head_dim], [kv_heads*head_dim]) instead of
+    # head by head.
+    qk_norm_whole: bool = False
+    score_cap: Optional[float] = None    # a scaled score s becomes cap * tanh(s / cap) before the softmax
 
 
 @dataclass(frozen=True)
@@ -140,11 +147,25 @@ class LatentAttentionSpec:
     o_proj: str
     position: Optional[Any] = None   # a spec that gives cosines and sines for rotary_dim / 2 neighbouring pairs
     window: Optional[int] = None
+    head_gate: Optional[str] = None  # tensor [heads, hidden]: head h's output is multiplied by sigmoid(row h of it . the mixer's input)
+
+
+@dataclass(frozen=True)
+class TokenShiftSpec:
+    """A mixer whose input h is first blended, channel by channel, with the input of the token before: h + (h_before - h) * w, with
+    `weight` [hidden] and h_before the row the request's previous token brought, before its own blending (zeros for a request's
+    first token).  `inner` is the spec of the mixer that reads the blended rows; it keeps the cache it would keep alone, and the
+    last row's h is kept per request beside it."""
+    kind: ClassVar[str] = "token_shift"
+    hidden_size: int
+    weight: str
+    inner: Any
 
 
 @dataclass(frozen=True)
 class SwiGluSpec:
-    """down( act(gate(x)) * up(x) ), no biases; act is SiLU, or the tanh form of GELU (`activation` = "gelu_tanh")."""
+    """down( act(gate(x)) * up(x) ), no biases; act is SiLU, or the tanh form of GELU (`activation` = "gelu_tanh"), or, as
+    "swish_clamped" with `activation_limit` L: g <- min(gate(x), L), u <- clamp(up(x), -L, L), down(g sigmoid(1.702 g) (u + 1))."""
     kind: ClassVar[str] = "swiglu"
     hidden_size: int
     intermediate_size: int
@@ -152,6 +173,7 @@ class SwiGluSpec:
     up_proj: str
     down_proj: str
     activation: str = "silu"
+    activation_limit: float = 0.0
 
 
 @dataclass(frozen=True)
@@ -244,8 +266,11 @@ class RoutedExpertsSpec:
     """A mixture of gated feed-forwards: `router` [experts, hidden] gives a logit per expert in 32-bit; the scores are their sigmoids
     (`score` = "sigmoid") or a softmax over all experts ("softmax"); the `top` experts with the largest scores serve the row.  The
     chosen scores, divided by their sum if `renormalize`, weigh each chosen expert's input (`weigh` = "input": the sum of
-    expert(w h)) or its output ("output": the sum of w expert(h)).  An expert is down(act(gate(a)) * up(a)) without biases.  `shared`,
-    a feed-forward spec of any kind, serves every row and is added."""
+    expert(w h)) or its output ("output": the sum of w expert(h)).  An expert is down(act(gate(a)) * up(a)) without biases (the
+    activations of `SwiGluSpec`, `activation_limit` with them).  `shared`, a feed-forward spec of any kind, serves every row and is
+    added; with `shared_gate` [1, hidden] it is multiplied by sigmoid(shared_gate . h) first, one number a row.  With `n_groups` > 1 the
+    experts form that many equal groups of neighbours, a group scores what its best expert scores, and only experts of the
+    `groups_kept` best groups can be chosen.  `renormalize_floor` is added to the sum the chosen scores are divided by."""
     kind: ClassVar[str] = "routed_experts"
     hidden_size: int
     intermediate_size: int
@@ -260,10 +285,20 @@ class RoutedExpertsSpec:
     weigh: str = "input"
     activation: str = "silu"
     shared: Optional[Any] = None
+    activation_limit: float = 0.0
+    shared_gate: Optional[str] = None
+    n_groups: int = 1
+    groups_kept: int = 1
+    renormalize_floor: float = 0.0
 
     def __post_init__(self):
         if not (len(self.gate_projs) == len(self.up_projs) == len(self.down_projs) == self.n_experts) or not 1 <= self.top <= self.n_experts:
             raise ValueError("routed experts: three matrices per expert, and 1 <= top <= experts")
+        if (self.n_groups < 1 or self.n_experts % self.n_groups or not 1 <= self.groups_kept <= self.n_groups
+                or self.top > self.groups_kept * (self.n_experts // self.n_groups)):
+            raise ValueError("routed experts: equal groups, of which 1 .. all are kept, with at least `top` experts in the kept ones")
+        if self.shared_gate is not None and self.shared is None:
+            raise ValueError("routed experts: a gate on the shared feed-forward needs a shared feed-forward")
 
 
 @dataclass(frozen=True)
@@ -341,6 +376,18 @@ class SoftCapSpec:
 
 
 @dataclass(frozen=True)
+class StreamAccessSpec:
+    """How one half of a layer uses the n copies x_0 .. x_(n-1) of the residual stream: it reads u = sum_s read[s] x_s, and with its
+    result y every copy becomes x_t <- sum_s mix[s, t] x_s + c * write[t] * y, all copies at once from the old ones (c the layer's
+    `residual_scale`).  Tensors `read` [n], `write` [n], `mix` [n, n], the matrix indexed [from, to]."""
+    kind: ClassVar[str] = "stream_access"
+    n_streams: int
+    read: str
+    write: str
+    mix: str
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One layer: which parts, and in which arrangement (`block`) they are wired."""
     mixer: Any
@@ -351,6 +398,11 @@ class LayerSpec:
     mixer_post_norm: Any = None      # "sandwich" blocks: a norm on what each half puts out, before it joins the residual stream
     feed_forward_post_norm: Any = None
     after: Tuple[Any, ...] = ()      # specs of parts that change the residual stream in place behind the block, in order (stream parts)
+    # "multistream" blocks (models that carry several copies of the residual stream): how each half reads and writes the copies,
+    # and what a half's result is multiplied by on its way into the stream
+    mixer_streams: Any = None
+    feed_forward_streams: Any = None
+    residual_scale: float = 1.0
 
 
 @dataclass(frozen=True)
@@ -378,6 +430,9 @@ class ModelSpec:
     ignorable_tensors: Tuple[str, ...] = field(default=())   # regular expressions of names a file may hold unused
     after_embedding: Tuple[Any, ...] = field(default=())     # row-transform specs applied, in order, to the rows of the token table
     after_head: Tuple[Any, ...] = field(default=())          # ... and to the logits
+    # Copies of the residual stream that the layers carry side by side (rows [n_streams * hidden]): all equal to the token rows at the
+    # start, added up before the final norm.  More than one needs blocks that know of them (`stream_aware`).
+    n_streams: int = 1
 
     def __post_init__(self):
         for i, e in enumerate(self.run_order):

@@ -12,6 +12,7 @@
 // The order of every sum depends on (pos, window, hd) only, so a row's result has the same bits
 // whatever else is in the batch and whichever pages hold its request.
 //
+// With `cap` > 0 a scaled score s becomes cap * tanh(s / cap) before the softmax.
 // With `sinks` [n_heads] the softmax's denominator also holds exp(sinks[h]): a score that has no key and no value (the
 // running maximum starts there and the running sum at 1).  With `gate` the head's output is multiplied by
 // sigmoid(gate[t * gate_stride + h]).
@@ -29,7 +30,7 @@ template <typename TQ, typename TC, typename TO>
 __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restrict__ q, const TC* __restrict__ cache, TO* __restrict__ out,
                                                             const int* __restrict__ pos, const int* __restrict__ slot,
                                                             const int* __restrict__ table, int table_stride, long page_stride,
-                                                            int page_size, int n_heads, int n_kv, int hd, int vd, int window, int chunk, float scale,
+                                                            int page_size, int n_heads, int n_kv, int hd, int vd, int window, int chunk, float scale, float cap,
                                                             const float* __restrict__ sinks, const float* __restrict__ gate, long gate_stride) {
     __shared__ float q_s[MAX_HD];
     __shared__ float p_s[64];
@@ -59,6 +60,7 @@ __global__ __launch_bounds__(64) void attention_exact_kernel(const TQ* __restric
             float dot = 0.f;
             for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], load_f32(cache, off + d), dot);
             s = dot * scale;
+            if (cap > 0.f) s = cap * tanhf(s / cap);
         }
         const float m_new = fmaxf(m, wave_max(s));
         const float p = valid ? expf(s - m_new) : 0.f;
@@ -97,19 +99,19 @@ GI_API int gi_attention_exact_max_head_size() { return MAX_HD; }
 
 GI_API int gi_attention_exact(const void* q, int q_dtype, const void* cache, int cache_dtype, void* out, int out_dtype, const int* pos,
                               const int* slot, const int* table, int table_stride, long page_stride, int page_size, int n_rows,
-                              int n_heads, int n_kv, int hd, int vd, int window, int chunk, float scale, const float* sinks, const float* gate,
+                              int n_heads, int n_kv, int hd, int vd, int window, int chunk, float scale, float cap, const float* sinks, const float* gate,
                               long gate_stride, hipStream_t stream) {
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_exact: bad head counts (%d rows, %d heads, %d kv heads)",
                n_rows, n_heads, n_kv);
     GI_REQUIRE(hd > 0 && hd <= MAX_HD, "attention_exact: head size %d is outside 1..%d", hd, MAX_HD);
     GI_REQUIRE(vd > 0 && vd <= MAX_HD, "attention_exact: value head size %d is outside 1..%d", vd, MAX_HD);
-    GI_REQUIRE(window >= 0 && chunk >= 0 && (gate == nullptr || gate_stride >= n_heads), "attention_exact: bad window, chunk or gate stride");
+    GI_REQUIRE(window >= 0 && chunk >= 0 && cap >= 0.f && (gate == nullptr || gate_stride >= n_heads), "attention_exact: bad window, chunk or gate stride");
     GI_REQUIRE(page_size > 0 && page_stride >= (long)n_kv * page_size * (hd + vd), "attention_exact: page stride %ld too small", page_stride);
     GI_REQUIRE((long)n_rows * n_heads < 2147483647L, "attention_exact: too many (row, head) pairs");
     const unsigned grid = (unsigned)(n_rows * n_heads);
 #define GO(TQ, TC, TO)                                                                                                          \
     attention_exact_kernel<TQ, TC, TO><<<grid, 64, 0, stream>>>((const TQ*)q, (const TC*)cache, (TO*)out, pos, slot, table, table_stride, \
-                                                                page_stride, page_size, n_heads, n_kv, hd, vd, window, chunk, scale, sinks, gate, gate_stride)
+                                                                page_stride, page_size, n_heads, n_kv, hd, vd, window, chunk, scale, cap, sinks, gate, gate_stride)
     if (q_dtype == GI_F32 && cache_dtype == GI_F32 && out_dtype == GI_F32) GO(float, float, float);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && out_dtype == GI_BF16) GO(bf16_t, bf16_t, bf16_t);
     else return gi_fail("attention_exact: dtypes (%d, %d, %d) must be all float32 or all bfloat16", q_dtype, cache_dtype, out_dtype);

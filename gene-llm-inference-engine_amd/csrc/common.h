@@ -47,6 +47,21 @@ __device__ __forceinline__ float load_f32(const bf16_t* p, size_t i) { return bf
 __device__ __forceinline__ void store_f32(float* p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void store_f32(bf16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
 
+// The gated feed-forwards' activations, act(gate) * up with the float32 products of a row:
+//   0  SiLU(g) * u
+//   1  the tanh form of GELU, 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))), times u
+//   2  both halves clamped first, g <- min(g, limit), u <- clamp(u, -limit, limit): g * sigmoid(1.702 g) * (u + 1)
+constexpr int GI_N_ACTIVATIONS = 3;
+__device__ __forceinline__ float gated_act(float g, float u, int act, float limit) {
+    if (act == 2) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g * (1.0f / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
+    }
+    if (act == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+    return g * (1.0f / (1.0f + expf(-g))) * u;
+}
+
 // A workgroup barrier that waits for this wave's LDS traffic only.  __syncthreads() also waits for every load
 // from global memory the wave has in flight, which undoes a prefetch into registers; use this one where the
 // barrier orders LDS reads and writes and nothing else.

@@ -416,12 +416,12 @@ GI_API int gi_rmsnorm_add(const float* y, const void* w, int w_dtype, float* x, 
 // Values may be blended with those another layer made of the same rows: with `v_other` [n_rows, ld_other] and `v_blend` (one
 // number on the device), v <- (1 - blend) v + blend v_other is what goes into the page; `v_keep` [n_rows, ld_keep], if given, gets
 // this layer's values (with their bias, before any blending) for such a reader.
-// `flags`: NRS_NEIGHBOURS turns the pairs (2i, 2i + 1), i < rot/2, instead (angle i for pair i); NRS_UNIT_RMS divides every query and
+// `flags`: NRS_NORM_ALL takes the norm over all heads of the projection at once, with weights [heads * hd] ([kv heads * hd]); NRS_NEIGHBOURS turns the pairs (2i, 2i + 1), i < rot/2, instead (angle i for pair i); NRS_UNIT_RMS divides every query and
 // key head by its root mean square without weights (q_norm and k_norm must then be absent); NRS_NORM_LAST takes the norm, of
 // either form, behind the rotation instead of in front of it.  `v_scale` multiplies the values on their way into the pages (the
 // attention's result is linear in them: a layer that weighs its attention's result can weigh the values instead).
 constexpr int NRS_MAX_HD = 512;
-constexpr int NRS_NEIGHBOURS = 1, NRS_UNIT_RMS = 2, NRS_NORM_LAST = 4;
+constexpr int NRS_NEIGHBOURS = 1, NRS_UNIT_RMS = 2, NRS_NORM_LAST = 4, NRS_NORM_ALL = 8;
 
 template <typename TQ, typename TC, typename TW>
 __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
@@ -463,7 +463,18 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
         ss = fmaf(x, x, ss);
     }
     const bool normed = w != nullptr || (flags & NRS_UNIT_RMS), norm_last = normed && (flags & NRS_NORM_LAST);
-    const float r = normed ? 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps) : 1.0f;      // (a rotation keeps the sum of squares: the same number in front of it and behind it)
+    int span = hd;
+    if (normed && (flags & NRS_NORM_ALL)) {          // one norm over all heads of the projection: every head's wave sums the whole row, in the same order
+        span = (is_q ? n_heads : n_kv) * hd;
+        const float* all = src - h * hd;
+        ss = 0.f;
+        for (int d = lane; d < span; d += 64) {
+            const float x = bias ? all[d] + bias[d] : all[d];
+            ss = fmaf(x, x, ss);
+        }
+        w = w != nullptr ? w + h * hd : w;
+    }
+    const float r = normed ? 1.0f / sqrtf(wave_sum(ss) / (float)span + eps) : 1.0f;      // (a rotation keeps the sum of squares: the same number in front of it and behind it)
     if (normed && !norm_last) {
         for (int d = lane; d < hd; d += 64) s[d] = w != nullptr ? load_f32(w, d) * (r * s[d]) : r * s[d];
     }
@@ -529,21 +540,20 @@ GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, lo
 // h[t, i] = act(gu[t, i]) * gu[t, inter + i]; act 0: SiLU, 1: the tanh form of GELU,
 // 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
 template <typename TO>
-__global__ void act_mul_kernel(const float* __restrict__ gu, TO* __restrict__ h, int inter, size_t n, int act) {
+__global__ void act_mul_kernel(const float* __restrict__ gu, TO* __restrict__ h, int inter, size_t n, int act, float limit) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const size_t t = i / inter, c = i % inter;
     const float g = gu[t * 2 * inter + c], u = gu[t * 2 * inter + inter + c];
-    const float a = act == 0 ? g * (1.0f / (1.0f + expf(-g))) : 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
-    store_f32(h, i, a * u);
+    store_f32(h, i, gated_act(g, u, act, limit));
 }
 
-GI_API int gi_act_mul(const float* gate_up, void* h, int h_dtype, int n_rows, int inter, int act, hipStream_t stream) {
-    GI_REQUIRE(n_rows > 0 && inter > 0 && (act == 0 || act == 1), "act_mul: n_rows %d and inter %d must be positive, the activation 0 or 1", n_rows, inter);
+GI_API int gi_act_mul(const float* gate_up, void* h, int h_dtype, int n_rows, int inter, int act, float limit, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && inter > 0 && act >= 0 && act < GI_N_ACTIVATIONS, "act_mul: n_rows %d and inter %d must be positive, the activation one of the known", n_rows, inter);
     const size_t n = (size_t)n_rows * inter;
     const unsigned blocks = (unsigned)((n + 255) / 256);
-    if (h_dtype == GI_F32) act_mul_kernel<float><<<blocks, 256, 0, stream>>>(gate_up, (float*)h, inter, n, act);
-    else if (h_dtype == GI_BF16) act_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>(gate_up, (bf16_t*)h, inter, n, act);
+    if (h_dtype == GI_F32) act_mul_kernel<float><<<blocks, 256, 0, stream>>>(gate_up, (float*)h, inter, n, act, limit);
+    else if (h_dtype == GI_BF16) act_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>(gate_up, (bf16_t*)h, inter, n, act, limit);
     else return gi_fail("act_mul: unknown dtype %d", h_dtype);
     GI_CHECK_LAUNCH("act_mul");
     return 0;

@@ -24,25 +24,17 @@
 
 namespace {
 
-__device__ __forceinline__ float act_of(float z, int act) {
-    return act == 1 ? 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))) : z / (1.0f + expf(-z));
-}
-
 constexpr int ROUTE_PER_LANE = 16;      // experts a lane looks at: up to 1024 experts
 
-// One wave per row.  score_kind 0: sigmoid, 1: softmax over all experts.
-__global__ __launch_bounds__(64) void route_top_kernel(const float* __restrict__ logits, long ld, int n_experts, int top, int score_kind, int renormalize,
-                                                      int* __restrict__ ids, float* __restrict__ weights) {
-    const size_t t = blockIdx.x;
-    const int lane = threadIdx.x;
-    float z[ROUTE_PER_LANE];
+// What the router makes of a row's logits (z: this lane's experts lane, lane + 64, ...; -inf beyond the last): the scores
+// (score_kind 0: sigmoid, 1: softmax over all experts), the `top` largest (the lower index wins a tie), optionally divided by
+// their sum + floor.  With n_groups > 1 the experts form that many equal groups of neighbours, a group scores what its best
+// expert scores, and only experts of the `keep` best groups can be chosen (the lower group wins a tie).
+__device__ __forceinline__ void choose_experts(float (&z)[ROUTE_PER_LANE], int lane, size_t t, int n_experts, int top, int score_kind, int renormalize, float floor,
+                                               int n_groups, int keep, int* __restrict__ ids, float* __restrict__ weights) {
     float biggest = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < ROUTE_PER_LANE; ++i) {
-        const int e = lane + 64 * i;
-        z[i] = e < n_experts ? logits[t * ld + e] : -INFINITY;
-        biggest = fmaxf(biggest, z[i]);
-    }
+    for (int i = 0; i < ROUTE_PER_LANE; ++i) biggest = fmaxf(biggest, z[i]);
     float denominator = 1.0f;
     if (score_kind == 1) {
         biggest = wave_max(biggest);
@@ -50,6 +42,33 @@ __global__ __launch_bounds__(64) void route_top_kernel(const float* __restrict__
 #pragma unroll
         for (int i = 0; i < ROUTE_PER_LANE; ++i) s += lane + 64 * i < n_experts ? expf(z[i] - biggest) : 0.f;
         denominator = wave_sum(s);
+    }
+    if (n_groups > 1 && keep < n_groups) {
+        const int per = n_experts / n_groups;
+        unsigned kept = 0, taken = 0;                   // bit i: expert lane + 64 i lies in a group that is kept / has been looked at
+        for (int k = 0; k < keep; ++k) {
+            float best = -INFINITY;
+            int at = 0x7fffffff;
+#pragma unroll
+            for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+                if (!((taken >> i) & 1u) && z[i] > best) best = z[i], at = lane + 64 * i;
+            }
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ob = __shfl_xor(best, off, 64);
+                const int oa = __shfl_xor(at, off, 64);
+                if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
+            }
+            const int g = at / per;
+#pragma unroll
+            for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+                if ((lane + 64 * i) / per == g) kept |= 1u << i, taken |= 1u << i;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+            if (!((kept >> i) & 1u)) z[i] = -INFINITY;
+        }
     }
     float total = 0.f, mine = 0.f;
     int my_id = 0;
@@ -76,15 +95,29 @@ __global__ __launch_bounds__(64) void route_top_kernel(const float* __restrict__
     }
     if (lane < top) {
         ids[t * top + lane] = my_id;
-        weights[t * top + lane] = renormalize ? mine / total : mine;
+        weights[t * top + lane] = renormalize ? mine / (total + floor) : mine;
     }
+}
+
+// One wave per row.
+__global__ __launch_bounds__(64) void route_top_kernel(const float* __restrict__ logits, long ld, int n_experts, int top, int score_kind, int renormalize,
+                                                      float floor, int n_groups, int keep, int* __restrict__ ids, float* __restrict__ weights) {
+    const size_t t = blockIdx.x;
+    const int lane = threadIdx.x;
+    float z[ROUTE_PER_LANE];
+#pragma unroll
+    for (int i = 0; i < ROUTE_PER_LANE; ++i) {
+        const int e = lane + 64 * i;
+        z[i] = e < n_experts ? logits[t * ld + e] : -INFINITY;
+    }
+    choose_experts(z, lane, t, n_experts, top, score_kind, renormalize, floor, n_groups, keep, ids, weights);
 }
 
 // One wave per (row, choice, output j): both dot products over the row, the lanes' shares of k interleaved.
 template <typename TW, typename TA, typename TO>
 __global__ __launch_bounds__(256) void experts_gate_up_kernel(const TA* __restrict__ h, long ldh, const TW* __restrict__ w_gate, const TW* __restrict__ w_up,
                                                              const int* __restrict__ ids, const float* __restrict__ weights, int weigh_input,
-                                                             int top, TO* __restrict__ mid, long ldm, int width, int ff, int act, int group) {
+                                                             int top, TO* __restrict__ mid, long ldm, int width, int ff, int act, float limit, int group) {
     const size_t item = blockIdx.x;                     // (row * top + choice)
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int j = blockIdx.y * 4 + wave;
@@ -104,7 +137,7 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const TA* __restri
     }
     sg = wave_sum(sg);
     su = wave_sum(su);
-    if (lane == 0) store_f32(mid + item * ldm, j, act_of(sg, act) * su);
+    if (lane == 0) store_f32(mid + item * ldm, j, gated_act(sg, su, act, limit));
 }
 
 template <typename TW, typename TM>
@@ -134,7 +167,7 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const TM* __restrict_
 constexpr int ROUTE_MAX_EXPERTS = 64 * ROUTE_PER_LANE;
 template <typename TA, typename TW>
 __global__ __launch_bounds__(256) void route_rows_kernel(const TA* __restrict__ h, long ldh, const TW* __restrict__ router, long ldr, int width, int n_experts, int top,
-                                                        int score_kind, int renormalize, int* __restrict__ ids, float* __restrict__ weights,
+                                                        int score_kind, int renormalize, float floor, int n_groups, int keep, int* __restrict__ ids, float* __restrict__ weights,
                                                         float* __restrict__ logits_out, long ldl) {
     __shared__ float zs[ROUTE_MAX_EXPERTS];
     const size_t t = blockIdx.x;
@@ -163,48 +196,12 @@ __global__ __launch_bounds__(256) void route_rows_kernel(const TA* __restrict__ 
     __syncthreads();
     if (wave != 0) return;
     float z[ROUTE_PER_LANE];
-    float biggest = -INFINITY;
 #pragma unroll
     for (int i = 0; i < ROUTE_PER_LANE; ++i) {
         const int e = lane + 64 * i;
         z[i] = e < n_experts ? zs[e] : -INFINITY;
-        biggest = fmaxf(biggest, z[i]);
     }
-    float denominator = 1.0f;
-    if (score_kind == 1) {
-        biggest = wave_max(biggest);
-        float s = 0.f;
-#pragma unroll
-        for (int i = 0; i < ROUTE_PER_LANE; ++i) s += lane + 64 * i < n_experts ? expf(z[i] - biggest) : 0.f;
-        denominator = wave_sum(s);
-    }
-    float total = 0.f, mine = 0.f;
-    int my_id = 0;
-    for (int k = 0; k < top; ++k) {
-        float best = -INFINITY;
-        int at = 0x7fffffff;
-#pragma unroll
-        for (int i = 0; i < ROUTE_PER_LANE; ++i) {
-            if (z[i] > best) best = z[i], at = lane + 64 * i;
-        }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ob = __shfl_xor(best, off, 64);
-            const int oa = __shfl_xor(at, off, 64);
-            if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
-        }
-        const float score = score_kind == 1 ? expf(best - biggest) / denominator : 1.0f / (1.0f + expf(-best));
-        total += score;
-        if (lane == k) mine = score, my_id = at;
-#pragma unroll
-        for (int i = 0; i < ROUTE_PER_LANE; ++i) {
-            if (lane + 64 * i == at) z[i] = -INFINITY;
-        }
-    }
-    if (lane < top) {
-        ids[t * top + lane] = my_id;
-        weights[t * top + lane] = renormalize ? mine / total : mine;
-    }
+    choose_experts(z, lane, t, n_experts, top, score_kind, renormalize, floor, n_groups, keep, ids, weights);
 }
 
 constexpr int EXPERT_TILE = 128;          // rows of a tile of the grouped product
@@ -282,24 +279,30 @@ __global__ __launch_bounds__(256) void experts_combine_kernel(const float* __res
 
 }  // namespace
 
-GI_API int gi_route_top(const float* logits, long ld, int n_rows, int n_experts, int top, int score_kind, int renormalize, int* ids, float* weights, hipStream_t stream) {
+static int groups_fit(int n_experts, int top, int n_groups, int keep) {
+    return n_groups >= 1 && n_experts % n_groups == 0 && keep >= 1 && keep <= n_groups && top <= keep * (n_experts / n_groups);
+}
+
+GI_API int gi_route_top(const float* logits, long ld, int n_rows, int n_experts, int top, int score_kind, int renormalize, float floor, int n_groups, int keep,
+                        int* ids, float* weights, hipStream_t stream) {
+    GI_REQUIRE(groups_fit(n_experts, top, n_groups, keep), "route_top: %d experts in %d groups of which %d are kept cannot give %d a row", n_experts, n_groups, keep, top);
     GI_REQUIRE(n_rows > 0 && n_experts > 0 && n_experts <= 64 * ROUTE_PER_LANE && top > 0 && top <= n_experts && top <= 64 && ld >= n_experts && (score_kind == 0 || score_kind == 1),
                "route_top: bad sizes (rows %d, experts %d, top %d)", n_rows, n_experts, top);
-    route_top_kernel<<<n_rows, 64, 0, stream>>>(logits, ld, n_experts, top, score_kind, renormalize, ids, weights);
+    route_top_kernel<<<n_rows, 64, 0, stream>>>(logits, ld, n_experts, top, score_kind, renormalize, floor, n_groups, keep, ids, weights);
     GI_CHECK_LAUNCH("route_top");
     return 0;
 }
 
 GI_API int gi_experts_gate_up(const void* h, int h_dtype, long ldh, const void* w_gate, const void* w_up, int w_dtype, const int* ids, const float* weights,
-                              int weigh_input, void* mid, int mid_dtype, long ldm, int n_rows, int top, int width, int ff, int act, int group, hipStream_t stream) {
-    GI_REQUIRE(n_rows > 0 && top > 0 && top <= 65535 && width > 0 && ff > 0 && ldh >= width && ldm >= ff && (act == 0 || act == 1) && (long)n_rows * top < (1l << 31)
+                              int weigh_input, void* mid, int mid_dtype, long ldm, int n_rows, int top, int width, int ff, int act, float limit, int group, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && top > 0 && top <= 65535 && width > 0 && ff > 0 && ldh >= width && ldm >= ff && act >= 0 && act < GI_N_ACTIVATIONS && (long)n_rows * top < (1l << 31)
                && (group == 0 ? w_up != nullptr : group > 0 && ff % group == 0),
                "experts_gate_up: bad sizes (rows %d, top %d, width %d, ff %d)", n_rows, top, width, ff);
     dim3 grid(n_rows * top, (ff + 3) / 4);
     GI_REQUIRE(grid.y <= 65535, "experts_gate_up: experts too wide");
 #define LAUNCH(TW, TA, TO)                                                                                                                      \
     experts_gate_up_kernel<TW, TA, TO><<<grid, 256, 0, stream>>>((const TA*)h, ldh, (const TW*)w_gate, (const TW*)w_up, ids, weights, weigh_input, \
-                                                                 top, (TO*)mid, ldm, width, ff, act, group)
+                                                                 top, (TO*)mid, ldm, width, ff, act, limit, group)
     if (w_dtype == GI_BF16 && h_dtype == GI_BF16 && mid_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
     else if (w_dtype == GI_F32 && h_dtype == GI_F32 && mid_dtype == GI_F32) LAUNCH(float, float, float);
     else if (w_dtype == GI_BF16 && h_dtype == GI_F32 && mid_dtype == GI_F32) LAUNCH(bf16_t, float, float);
@@ -325,11 +328,12 @@ GI_API int gi_experts_down(const void* mid, int mid_dtype, long ldm, const void*
 }
 
 GI_API int gi_route_rows(const void* h, int h_dtype, long ldh, const void* router, int r_dtype, long ldr, int n_rows, int width, int n_experts, int top, int score_kind,
-                         int renormalize, int* ids, float* weights, float* logits, long ldl, hipStream_t stream) {
+                         int renormalize, float floor, int n_groups, int keep, int* ids, float* weights, float* logits, long ldl, hipStream_t stream) {
+    GI_REQUIRE(groups_fit(n_experts, top, n_groups, keep), "route_rows: %d experts in %d groups of which %d are kept cannot give %d a row", n_experts, n_groups, keep, top);
     GI_REQUIRE(n_rows > 0 && width > 0 && n_experts > 0 && n_experts <= ROUTE_MAX_EXPERTS && top > 0 && top <= n_experts && top <= 64 && ldh >= width && ldr >= width
                && (score_kind == 0 || score_kind == 1) && (logits == nullptr || ldl >= n_experts),
                "route_rows: bad sizes (rows %d, width %d, experts %d, top %d)", n_rows, width, n_experts, top);
-#define LAUNCH(TA, TW) route_rows_kernel<TA, TW><<<n_rows, 256, 0, stream>>>((const TA*)h, ldh, (const TW*)router, ldr, width, n_experts, top, score_kind, renormalize, ids, weights, logits, ldl)
+#define LAUNCH(TA, TW) route_rows_kernel<TA, TW><<<n_rows, 256, 0, stream>>>((const TA*)h, ldh, (const TW*)router, ldr, width, n_experts, top, score_kind, renormalize, floor, n_groups, keep, ids, weights, logits, ldl)
     if (h_dtype == GI_BF16 && r_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
     else if (h_dtype == GI_F32 && r_dtype == GI_F32) LAUNCH(float, float);
     else if (h_dtype == GI_F32 && r_dtype == GI_BF16) LAUNCH(float, bf16_t);

@@ -42,6 +42,13 @@ class DecoderModel:
         self.embedding = tensors[spec.embedding]
         self.lm_head = tensors[spec.lm_head]
         self.layers = [block_class(l.block)(l, tensors, dtype, device) for l in spec.layers]
+        self.n_streams = int(getattr(spec, "n_streams", 1))          # copies of the residual stream the layers carry side by side
+        if self.n_streams > 1:
+            for l, layer in zip(spec.layers, self.layers):
+                if not getattr(layer, "stream_aware", False) or getattr(layer, "n_streams", 1) != self.n_streams:
+                    raise ValueError(f"the model carries {self.n_streams} copies of the residual stream, which a '{l.block}' layer does not (or not as many)")
+            if any(l.after for l in spec.layers) or any(e.before is not None for e in spec.run_order):
+                raise ValueError("parts between the layers change one residual stream, not several copies of it")
         self.final_norm = norm_class(spec.final_norm)(spec.final_norm, tensors, dtype, device)
         self.head_in_dtype = activation_dtype_for(self.lm_head, dtype)
         self.head = _Head(self.lm_head, self.head_in_dtype)
@@ -85,6 +92,8 @@ class DecoderModel:
             trace("embedding", -1, x)
         if self.keeps_token_rows:
             ctx.memo["token_rows"] = x.clone()
+        if self.n_streams > 1:            # every copy starts as the token rows
+            x = ops.streams_spread(x, torch.empty((ctx.n_rows, self.n_streams * self.spec.hidden_size), dtype=torch.float32, device=self.device), self.n_streams)
         for i, entry in enumerate(self.run_order):
             ctx.trace = None if trace is None else (lambda tag, rows, i=i: trace(tag, i, rows))
             layer, extras = self.layers[entry.layer], self.after_layer[entry.layer]
@@ -110,6 +119,8 @@ class DecoderModel:
         ctx.trace = None
         if n_logit_rows == 0:
             return None
+        if self.n_streams > 1:            # the copies are added up before the final norm
+            x = ops.streams_norm_shift(x, self.n_streams, torch.empty((ctx.n_rows, self.spec.hidden_size), dtype=torch.float32, device=self.device))
         logits = torch.empty((n_logit_rows, self.spec.vocab_size), dtype=torch.float32, device=self.device)
         if handed is not None and handed.norm is self.final_norm and ctx.every_row_wanted:
             normed = handed
@@ -157,6 +168,13 @@ def load_model(folder, dtype="bfloat16", device="cuda:0") -> DecoderModel:
     configuration is chosen by config.json."""
     dtype = compute_dtype(dtype)
     config = read_config(folder)
+    if hasattr(config, "fit_to_tensors"):          # an architecture some of whose parts a folder may lack looks at the tensors' names
+        from ..weights.safetensors_io import SafetensorsFile
+        st = SafetensorsFile(Path(folder) / "model.safetensors")
+        try:
+            config = config.fit_to_tensors(list(st.entries))
+        finally:
+            st.close()
     spec = config.model_spec()
     tensors = load_tensors(folder, model_tensor_needs(spec), dtype, device, spec.ignorable_tensors)
     model = DecoderModel(spec, tensors, dtype, device)

@@ -35,7 +35,7 @@ _SIGNATURES = {
     "gi_softcap_rows": [c_void_p, c_int, c_int, c_long, c_float, c_void_p],
     "gi_gemm_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gi_attention_exact": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_void_p, c_void_p, c_long, c_void_p],
     "gi_rmsnorm_add": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_long, c_long, c_void_p],
     "gi_rmsnorm_add_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_long, c_long, c_long, c_void_p],
     "gi_norm_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int,
@@ -51,9 +51,9 @@ _SIGNATURES = {
     "gi_ssm_tail": [c_void_p, c_long, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p],
     "gi_ssm_scan": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                     c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
-    "gi_route_top": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
-    "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "gi_route_rows": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
+    "gi_route_top": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    "gi_route_rows": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
     "gi_experts_place": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "gi_experts_gather": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_void_p],
     "gi_experts_combine": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_int, c_void_p],
@@ -71,7 +71,13 @@ _SIGNATURES = {
                                  c_float, c_int, c_void_p],
     "gi_latent_attention_tiles_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     "gi_latent_queries": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
-    "gi_act_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+    "gi_act_mul": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_void_p],
+    "gi_streams_spread": [c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
+    "gi_streams_norm_shift": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_long,
+                              c_int, c_int, c_void_p],
+    "gi_streams_write": [c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_float, c_int, c_void_p],
+    "gi_head_gate": [c_void_p, c_int, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
+    "gi_add_rows_gated": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_void_p],
     "gi_segments": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],
     "gi_mlstm_scan": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_int, c_void_p,
                       c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -137,6 +143,8 @@ def lib():
         l.gi_latent_attention_tiles_supports.restype = c_int
         l.gi_latent_attention_tiles_prepare.argtypes = []
         l.gi_latent_attention_tiles_prepare.restype = c_int
+        l.gi_streams_max.argtypes = []
+        l.gi_streams_max.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
         l.gi_probe_mfma_flops.restype = c_long
         _lib = l
@@ -457,12 +465,14 @@ def _check_paged(cache, table, what):
 
 
 def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None, *, page_size=None, value_dim=None,
-                    chunk=None, sinks=None, gate=None):
+                    chunk=None, sinks=None, gate=None, cap=None):
     """Each row attends over its request's cached keys up to its own position, no further back than `window` positions and not
     beyond the start of its own chunk of `chunk` positions.  value_dim: channels of a value head (hd if not given); sinks:
     float32 [heads], a score per head that joins the softmax's denominator only; gate: float32 [n, >= heads] (unit inner
-    stride), head h's output is multiplied by sigmoid(gate[t, h])."""
+    stride), head h's output is multiplied by sigmoid(gate[t, h]); cap: a scaled score s becomes cap * tanh(s / cap)."""
     _dev(q, cache, out, positions, slots, table, sinks, gate)
+    if cap is not None and not cap > 0:
+        raise KernelError("attention: the scores' cap must be positive")
     n = q.shape[0]
     vd = int(value_dim or hd)
     if not (q.shape == (n, n_heads * hd) and q.is_contiguous() and out.shape == (n, n_heads * vd) and out.is_contiguous()):
@@ -481,7 +491,7 @@ def attention_exact(q, cache, out, positions, slots, table, n_heads, n_kv, hd, w
     _call("gi_attention_exact", q.data_ptr(), _code(q, "attention: q"), cache.data_ptr(), _code(cache, "attention: cache"), out.data_ptr(),
           _code(out, "attention: out"), positions.data_ptr(), slots.data_ptr(), table.data_ptr(), table.stride(0), cache.stride(0),
           page_size, n, n_heads, n_kv, hd, vd, int(window or 0), int(chunk or 0), float(scale if scale is not None else hd ** -0.5),
-          _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0, _stream())
+          float(cap or 0.0), _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0, _stream())
     return out
 
 
@@ -512,7 +522,7 @@ def rmsnorm_add_norm(y, weight, eps, x, next_weight, next_eps, out):
 
 
 def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, positions, slots, table, q_out, cache, page_size, n_heads, n_kv, hd, vd,
-                    biases=None, blend=None, keep=None, neighbours=False, unit_rms=False, norm_last=False, v_scale=1.0):
+                    biases=None, blend=None, keep=None, neighbours=False, unit_rms=False, norm_last=False, v_scale=1.0, norm_all=False):
     """The general form of `rope_store`: every query and key head is first RMS-normed with q_norm / k_norm [hd] (None: not), then
     the pairs (i, i + rotary_dim/2) of its first rotary_dim channels are turned (cos, sin float32 [n, rotary_dim/2]; None: not);
     queries go to q_out, keys and the values (vd channels a head) into the cache's pages.  k None: the pages are another layer's.
@@ -521,7 +531,8 @@ def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, position
     the same rows), weight one float32 number on the device.  keep: float32 [n, kv_heads*vd], gets this layer's values (with
     their bias, before any blending).  neighbours: the pairs turned are (2i, 2i + 1).  unit_rms: every query and key head is divided
     by its root mean square (eps inside the root), without weights.  norm_last: the heads' norm comes behind the rotation.
-    v_scale: multiplies the values on their way into the pages."""
+    v_scale: multiplies the values on their way into the pages.  norm_all: q_norm is [heads*hd] and k_norm [kv_heads*hd], and the norm is
+    taken over all heads of a projection at once."""
     if unit_rms and (q_norm is not None or k_norm is not None):
         raise KernelError("norm_rope_store: heads divided by their root mean square have no norm weights")
     _dev(q, k, v, q_norm, k_norm, cos, sin, positions, slots, table, q_out, cache)
@@ -547,10 +558,10 @@ def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, position
             if not (t.dtype == torch.float32 and t.shape == (n, half) and t.is_contiguous()):
                 raise KernelError("norm_rope_store: cos/sin must be float32 [n, rotary_dim/2]")
     norm_code = None
-    for w in (q_norm, k_norm):
+    for w, heads in ((q_norm, n_heads), (k_norm, n_kv)):
         if w is not None:
-            if not (w.shape == (hd,) and w.is_contiguous() and (norm_code is None or norm_code == _code(w, "norm_rope_store: norm"))):
-                raise KernelError("norm_rope_store: the heads' norm weights must be [hd], of one dtype")
+            if not (w.shape == ((heads * hd,) if norm_all else (hd,)) and w.is_contiguous() and (norm_code is None or norm_code == _code(w, "norm_rope_store: norm"))):
+                raise KernelError("norm_rope_store: the norm weights must be [hd] (over all heads at once: [heads*hd]), of one dtype")
             norm_code = _code(w, "norm_rope_store: norm")
     if k is not None:
         if not (k.dtype == torch.float32 and k.shape == (n, n_kv * hd) and k.stride(1) == 1 and v.dtype == torch.float32 and v.shape == (n, n_kv * vd) and v.stride(1) == 1):
@@ -566,7 +577,7 @@ def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, position
           slots.data_ptr(), _ptr(table) if k is not None else None, table.stride(0) if k is not None else 0, q_out.data_ptr(),
           _code(q_out, "norm_rope_store: q_out"), _ptr(cache) if k is not None else None, cache_code, cache.stride(0) if k is not None else 0,
           int(page_size), n, n_heads, n_kv, hd, vd, _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), _ptr(other), other.stride(0) if other is not None else 0,
-          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, (1 if neighbours else 0) | (2 if unit_rms else 0) | (4 if norm_last else 0), float(v_scale), _stream())
+          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, (1 if neighbours else 0) | (2 if unit_rms else 0) | (4 if norm_last else 0) | (8 if norm_all else 0), float(v_scale), _stream())
 
 
 def xielu(x, out, params):
@@ -582,18 +593,22 @@ def xielu(x, out, params):
     return out
 
 
-ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swish_clamped": 2}
+# "swish_clamped" takes a number, `limit`: both halves are clamped first, g <- min(g, limit), u <- clamp(u, -limit, limit), and the
+# result is g * sigmoid(1.702 g) * (u + 1).
+FUSED_GATE_ACTIVATIONS = ("silu", "gelu_tanh")        # those the matrix-core products apply in their own last step
 
 
-def act_mul(gate_up, out, activation="silu"):
-    """out[t, i] = act(gate_up[t, i]) * gate_up[t, inter + i]; act "silu" or "gelu_tanh" (the tanh form of GELU)."""
+def act_mul(gate_up, out, activation="silu", limit=0.0):
+    """out[t, i] = act(gate_up[t, i]) * gate_up[t, inter + i]; act "silu", "gelu_tanh" (the tanh form of GELU), or the clamped form
+    "swish_clamped" with its `limit` (see `ACTIVATIONS`)."""
     _dev(gate_up, out)
     n, inter = out.shape
     if activation not in ACTIVATIONS:
         raise KernelError(f"act_mul: unknown activation {activation!r}; known: {', '.join(ACTIVATIONS)}")
     if not (gate_up.dtype == torch.float32 and gate_up.shape == (n, 2 * inter) and gate_up.is_contiguous() and out.is_contiguous()):
         raise KernelError("act_mul: gate_up must be float32 [n, 2*inter], out contiguous")
-    _call("gi_act_mul", gate_up.data_ptr(), out.data_ptr(), _code(out, "act_mul: out"), n, inter, ACTIVATIONS[activation], _stream())
+    _call("gi_act_mul", gate_up.data_ptr(), out.data_ptr(), _code(out, "act_mul: out"), n, inter, ACTIVATIONS[activation], float(limit), _stream())
     return out
 
 
@@ -1089,17 +1104,18 @@ def attention(q, cache, out, ctx, table, n_heads, n_kv, hd, window=None):
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window)
 
 
-def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size, value_dim=None, window=None, chunk=None, scale=None, sinks=None, gate=None):
+def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size, value_dim=None, window=None, chunk=None, scale=None, sinks=None, gate=None,
+                      cap=None):
     """Attention of a step's rows for layers with any of: value heads of another size, a scale of their own, a mask cut into
-    chunks, sinks, a gate per head."""
+    chunks, sinks, a gate per head, capped scores."""
     vd = int(value_dim or hd)
-    if (vd == hd and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+    if (cap is None and vd == hd and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
             and (gate is None or gate.dtype == torch.float32)):
         plan = _plan_of(ctx)
         if (not plan.n_tiles or attention_bf16_supports(hd, page_size, True)) and (not plan.n_decode or attention_bf16_supports(hd, page_size, False)):
             return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, chunk=chunk, sinks=sinks, gate=gate)
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, page_size=page_size,
-                           value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate)
+                           value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate, cap=cap)
 
 
 # Up to so many rows the decode kernel rotates and writes the pages itself.  It saves the rotation kernel's launch wherever the
@@ -1596,9 +1612,17 @@ EXPERT_TILE_ROWS = 128         # rows of a tile of the product for grouped rows 
 EXPERTS_GROUPED_FROM = 8       # (row, choice) items from which the experts' rows are grouped for the matrix cores
 
 
-def route_top(logits, top, ids, weights, score="sigmoid", renormalize=False):
+def _router_groups(what, n_experts, top, groups):
+    n_groups, keep = (1, 1) if groups is None else (int(groups[0]), int(groups[1]))
+    if not (n_groups >= 1 and n_experts % n_groups == 0 and 1 <= keep <= n_groups and top <= keep * (n_experts // n_groups)):
+        raise KernelError(f"{what}: {n_experts} experts in {n_groups} groups of which {keep} are kept cannot give {top} a row")
+    return n_groups, keep
+
+
+def route_top(logits, top, ids, weights, score="sigmoid", renormalize=False, groups=None, floor=0.0):
     """ids int32 [n, top], weights float32 [n, top]: per row the `top` experts with the largest scores (the lower index wins a tie)
-    and their scores, divided by their sum if `renormalize`."""
+    and their scores, divided by their sum + `floor` if `renormalize`.  groups = (count, keep): the experts form `count` equal groups
+    of neighbours, a group scores what its best expert scores, and only experts of the `keep` best groups can be chosen."""
     _dev(logits, ids, weights)
     n, n_experts = logits.shape
     _f32_rows(logits, "route_top: logits")
@@ -1608,7 +1632,8 @@ def route_top(logits, top, ids, weights, score="sigmoid", renormalize=False):
         raise KernelError(f"route_top: top {top} of {n_experts} experts is outside what the kernel takes")
     if not (ids.dtype == torch.int32 and ids.shape == (n, top) and ids.is_contiguous() and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()):
         raise KernelError("route_top: ids must be int32 [n, top] and weights float32 [n, top], contiguous")
-    _call("gi_route_top", logits.data_ptr(), logits.stride(0), n, n_experts, top, ROUTER_SCORES[score], 1 if renormalize else 0, ids.data_ptr(), weights.data_ptr(), _stream())
+    _call("gi_route_top", logits.data_ptr(), logits.stride(0), n, n_experts, top, ROUTER_SCORES[score], 1 if renormalize else 0, float(floor),
+          *_router_groups("route_top", n_experts, top, groups), ids.data_ptr(), weights.data_ptr(), _stream())
 
 
 def _expert_stack(w, rows, cols, what):
@@ -1616,7 +1641,7 @@ def _expert_stack(w, rows, cols, what):
         raise KernelError(f"{what} must be [experts, {rows}, {cols}], contiguous")
 
 
-def experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=True, activation="silu"):
+def experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=True, activation="silu", limit=0.0):
     """mid[(row, choice)] = act(W_gate[e] a) * (W_up[e] a), a = the row of h (times the choice's weight if `weigh_input`, stored as
     h's dtype), e = ids[row, choice]; one wave per output, for the few rows of decoding steps.  w_up None: w_gate is one stack
     [experts, 2 ff, width] of 16 gate rows, the 16 up rows of the same outputs, and so on (`interleave_gate_up` per expert)."""
@@ -1635,7 +1660,7 @@ def experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=True, activa
         raise KernelError("experts_gate_up: h [n, width], mid [n * top, ff], ids int32 and weights float32 [n, top] are needed")
     _call("gi_experts_gate_up", h.data_ptr(), _code(h, "experts_gate_up: h"), h.stride(0), w_gate.data_ptr(), _ptr(w_up), _code(w_gate, "experts_gate_up: weights"),
           ids.data_ptr(), weights.data_ptr(), 1 if weigh_input else 0, mid.data_ptr(), _code(mid, "experts_gate_up: mid"), mid.stride(0), n, top, width, ff,
-          ACTIVATIONS[activation], group, _stream())
+          ACTIVATIONS[activation], float(limit), group, _stream())
     return mid
 
 
@@ -1654,9 +1679,9 @@ def experts_down(mid, w_down, ids, weights, x, accumulate=True, weigh_output=Fal
     return x
 
 
-def route_rows(h, router, top, ids, weights, score="sigmoid", renormalize=False, logits=None):
+def route_rows(h, router, top, ids, weights, score="sigmoid", renormalize=False, logits=None, groups=None, floor=0.0):
     """The router's product and its choice in one launch: logits = h @ router.T with 32-bit sums in an order that the width alone
-    fixes, then as `route_top`.  logits: float32 [n, experts] to keep them in, or None."""
+    fixes, then as `route_top` (with its `groups` and `floor`).  logits: float32 [n, experts] to keep them in, or None."""
     _dev(h, router, ids, weights, logits)
     n, width = h.shape
     n_experts = router.shape[0]
@@ -1670,7 +1695,8 @@ def route_rows(h, router, top, ids, weights, score="sigmoid", renormalize=False,
     if logits is not None:
         _f32_rows(logits, "route_rows: logits", n, n_experts)
     _call("gi_route_rows", h.data_ptr(), _code(h, "route_rows: h"), h.stride(0), router.data_ptr(), _code(router, "route_rows: the router"), router.stride(0), n, width,
-          n_experts, top, ROUTER_SCORES[score], 1 if renormalize else 0, ids.data_ptr(), weights.data_ptr(), _ptr(logits), logits.stride(0) if logits is not None else 0, _stream())
+          n_experts, top, ROUTER_SCORES[score], 1 if renormalize else 0, float(floor), *_router_groups("route_rows", n_experts, top, groups), ids.data_ptr(), weights.data_ptr(),
+          _ptr(logits), logits.stride(0) if logits is not None else 0, _stream())
 
 
 def gemm_bf16_grouped(a, w, out, tile_group, gated=False):
@@ -1703,7 +1729,7 @@ def experts_grouped_supported(h, w_gate, w_up, w_down) -> bool:
     return width % 64 == 0 and ff % 64 == 0 and width >= 128 and 2 * ff >= 128 and h.stride(0) % 8 == 0 and h.data_ptr() % 16 == 0
 
 
-def routed_experts(h, w_gate, w_up, w_down, ids, weights, x, accumulate=True, weigh="input", activation="silu"):
+def routed_experts(h, w_gate, w_up, w_down, ids, weights, x, accumulate=True, weigh="input", activation="silu", limit=0.0):
     """x[row] (+)= sum over the row's choices of expert(a): the whole mixture behind the router's choice.  weigh "input": a = weight * h[row]
     (stored as h's dtype); "output": a = h[row] and the weight multiplies the expert's result.  w_up None: w_gate holds both (see
     `experts_gate_up`).  Few items, or 32-bit operands: every item walks its expert's matrices.  Many in bfloat16: the items' rows are
@@ -1713,7 +1739,7 @@ def routed_experts(h, w_gate, w_up, w_down, ids, weights, x, accumulate=True, we
     n, top = ids.shape
     n_experts, width = w_down.shape[0], w_down.shape[1]
     ff = w_down.shape[2]
-    if n * top >= EXPERTS_GROUPED_FROM and experts_grouped_supported(h, w_gate, w_up, w_down):
+    if n * top >= EXPERTS_GROUPED_FROM and activation in FUSED_GATE_ACTIVATIONS and experts_grouped_supported(h, w_gate, w_up, w_down):
         _dev(h, w_gate, w_down, ids, weights, x)
         _f32_rows(x, "routed_experts: x", n, width)
         if not (ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()
@@ -1737,6 +1763,94 @@ def routed_experts(h, w_gate, w_up, w_down, ids, weights, x, accumulate=True, we
         return x
     mid_dtype = torch.float32 if w_down.dtype == torch.float32 else h.dtype
     mid = torch.empty((n * top, ff), dtype=mid_dtype, device=h.device)
-    experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=weigh == "input", activation=activation)
+    experts_gate_up(h, w_gate, w_up, ids, weights, mid, weigh_input=weigh == "input", activation=activation, limit=limit)
     experts_down(mid, w_down, ids, weights, x, accumulate=accumulate, weigh_output=weigh == "output")
+    return x
+
+
+# ---------------------------------------------------------------- several copies of the residual stream, the row before a row
+def streams_max() -> int:
+    return lib().gi_streams_max()
+
+
+def streams_spread(x0, x, n_streams):
+    """Every one of the n copies in x [rows, n * width] <- x0 [rows, width] (float32)."""
+    _dev(x0, x)
+    rows, width = x0.shape
+    _f32_rows(x0, "streams_spread: the rows", rows, width)
+    _f32_rows(x, "streams_spread: the copies", rows, n_streams * width)
+    _call("gi_streams_spread", x0.data_ptr(), x0.stride(0), x.data_ptr(), x.stride(0), rows, n_streams, width, _stream())
+    return x
+
+
+def streams_norm_shift(x, n_streams, out, *, read=None, norm_weight=None, eps=0.0, shift=None, state=None, positions=None, slots=None, mode=1):
+    """x float32 [rows, n * width]: u = sum_s read[s] x_s (read None: the plain sum), h = norm_weight * u / sqrt(mean(u^2) + eps)
+    (norm_weight None: h = u), and, with `shift` float32 [width], out = h + (h_before - h) * shift with h_before the h of the
+    request's row before (zeros at position 0; the step's previous row, or the request's slot of `state` float32 [slots, width]).
+    mode 1 writes out, mode 2 lets every request's last row of the step write its h into its slot, 3 both: in one launch only if
+    every request brings one row."""
+    _dev(x, out, read, norm_weight, shift, state, positions, slots)
+    rows = x.shape[0]
+    width = x.shape[1] // n_streams
+    _f32_rows(x, "streams_norm_shift: x", rows, n_streams * width)
+    if not 1 <= n_streams <= streams_max():
+        raise KernelError(f"streams_norm_shift: 1 to {streams_max()} copies of the stream are taken, not {n_streams}")
+    if mode & 1 and not (out is not None and out.shape == (rows, width) and out.stride(1) == 1):
+        raise KernelError("streams_norm_shift: out must be [rows, width] with unit inner stride")
+    for v, n, what in ((read, n_streams, "the copies' weights"), (shift, width, "the blend's weights")):
+        if v is not None and not (v.dtype == torch.float32 and v.is_contiguous() and v.numel() == n):
+            raise KernelError(f"streams_norm_shift: {what} must be float32 [{n}]")
+    if norm_weight is not None and not (norm_weight.shape == (width,) and norm_weight.is_contiguous()):
+        raise KernelError("streams_norm_shift: the norm's weights must be [width]")
+    if shift is not None:
+        if not (state is not None and state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == width and state.stride(1) == 1):
+            raise KernelError("streams_norm_shift: the state must be float32 [slots, width]")
+        _i32(positions, "streams_norm_shift: positions", rows)
+        _i32(slots, "streams_norm_shift: slots", rows)
+    elif mode != 1:
+        raise KernelError("streams_norm_shift: without a blend there is no state to write")
+    _call("gi_streams_norm_shift", x.data_ptr(), x.stride(0), n_streams, width, _ptr(read), _ptr(norm_weight), _code(norm_weight, "streams_norm_shift: norm") if norm_weight is not None else F32,
+          float(eps), _ptr(shift), _ptr(state), state.stride(0) if state is not None else 0, _ptr(positions), _ptr(slots), _ptr(out) if mode & 1 else None,
+          _code(out, "streams_norm_shift: out") if out is not None else F32, out.stride(0) if out is not None else width, rows, int(mode), _stream())
+    return out
+
+
+def streams_write(x, n_streams, y, mix, write, mult=1.0):
+    """x float32 [rows, n * width] in place: copy t <- sum_s mix[s, t] copy_s + mult * write[t] * y, all copies at once from the old
+    ones; mix float32 [n, n] (None: every copy keeps itself), write float32 [n] (None: ones), y float32 [rows, width]."""
+    _dev(x, y, mix, write)
+    rows = x.shape[0]
+    width = x.shape[1] // n_streams
+    _f32_rows(x, "streams_write: x", rows, n_streams * width)
+    _f32_rows(y, "streams_write: y", rows, width)
+    if not 1 <= n_streams <= streams_max():
+        raise KernelError(f"streams_write: 1 to {streams_max()} copies of the stream are taken, not {n_streams}")
+    if mix is not None and not (mix.dtype == torch.float32 and mix.is_contiguous() and mix.shape == (n_streams, n_streams)):
+        raise KernelError("streams_write: the mixing matrix must be float32 [n, n]")
+    if write is not None and not (write.dtype == torch.float32 and write.is_contiguous() and write.numel() == n_streams):
+        raise KernelError("streams_write: the writing weights must be float32 [n]")
+    _call("gi_streams_write", x.data_ptr(), x.stride(0), n_streams, width, y.data_ptr(), y.stride(0), _ptr(mix), _ptr(write), float(mult), rows, _stream())
+    return x
+
+
+def head_gate(a, gate, n_heads, vd):
+    """a [rows, heads * vd] in place: head h of row t multiplied by sigmoid(gate[t, h]); gate float32 [rows, >= heads] (unit inner stride)."""
+    _dev(a, gate)
+    rows = a.shape[0]
+    if not (a.shape == (rows, n_heads * vd) and a.stride(1) == 1 and gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == rows and gate.shape[1] >= n_heads
+            and gate.stride(1) == 1):
+        raise KernelError("head_gate: a must be [rows, heads*vd] and the gates float32 [rows, heads], with unit inner stride")
+    _call("gi_head_gate", a.data_ptr(), _code(a, "head_gate: a"), a.stride(0), gate.data_ptr(), gate.stride(0), rows, n_heads, vd, _stream())
+    return a
+
+
+def add_rows_gated(x, y, g):
+    """x[t] += sigmoid(g[t]) * y[t]; x, y float32 [rows, width], g float32 [rows] (any stride)."""
+    _dev(x, y, g)
+    rows, width = x.shape
+    _f32_rows(x, "add_rows_gated: x", rows, width)
+    _f32_rows(y, "add_rows_gated: y", rows, width)
+    if not (g.dtype == torch.float32 and g.numel() == rows and g.dim() <= 2):
+        raise KernelError("add_rows_gated: the gates must be float32, one a row")
+    _call("gi_add_rows_gated", x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0), g.data_ptr(), g.stride(0), rows, width, _stream())
     return x

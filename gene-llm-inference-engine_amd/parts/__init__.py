@@ -3,7 +3,7 @@ from .base import (FeedForward, LayerCache, Mixer, Norm, Part, PositionEncoding,
                    feed_forward_class, mixer_class, norm_class, position_class, register_block, register_feed_forward,
                    register_mixer, register_norm, register_position_encoding, register_row_transform, register_stream_part,
                    row_transform_class, stream_part_class, weight_bytes, weight_tensors)
-from . import norm, rope, attention, mlp, mlstm, delta, latent, selective, side_by_side, experts, stream, block, transform          # registers the built-in kinds
+from . import norm, rope, attention, mlp, mlstm, delta, latent, selective, side_by_side, experts, stream, block, multistream, transform          # registers the built-in kinds
 from .linear import linear, linear_onto
 from .attention import qkv_rotate_store_attend
 from ..weights.loader import TensorNeed

@@ -86,8 +86,8 @@ def _pad_rows(w, multiple=16):
 
 class Attention(Mixer):
     """Plain (Llama) attention takes the kernels chosen in `qkv_rotate_store_attend`.  A spec that names any of the further
-    features (value heads of another size, a scale of its own, a mask cut into chunks, sinks, norms on query and key heads, a
-    gate per head, a rotation of a part of the head) takes the general path: one product with [q; k; v; head gates], one kernel
+    features (value heads of another size, a scale of its own, a mask cut into chunks, sinks, norms on query and key heads or over
+    the whole projections, a gate per head, a rotation of a part of the head, capped scores) takes the general path: one product with [q; k; v; head gates], one kernel
     that norms, turns and stores, and the attention kernel that knows all of these."""
     accepts_deferred_norm = True      # its input goes into `linear` only
     hands_norm_on = True              # `forward` takes `then`, the norm that reads the residual next
@@ -121,6 +121,12 @@ class Attention(Mixer):
             if s.value_blend is not None and s.value_family is None:
                 raise ValueError("attention: a blend of values needs the family whose first layer's values are blended in")
             self.unit_rms = bool(getattr(s, "qk_unit_rms", False))
+            self.norm_whole = bool(getattr(s, "qk_norm_whole", False))
+            if self.norm_whole and (self.q_norm is None or (self.k_norm is None and s.k_proj is not None)):
+                raise ValueError("attention: a norm over the whole query and key projections needs its weights")
+            self.score_cap = getattr(s, "score_cap", None)
+            if self.score_cap is not None and not self.score_cap > 0:
+                raise ValueError("attention: the scores' cap must be positive")
             if self.unit_rms and (self.q_norm is not None or self.k_norm is not None):
                 raise ValueError("attention: heads divided by their root mean square have no norm weights")
             if self.position is not None and hasattr(self.position, "pair_tables") and self.position.rotary_dim > s.head_dim:
@@ -139,7 +145,7 @@ class Attention(Mixer):
     @staticmethod
     def _is_general(s) -> bool:
         return (s.k_proj is None or any(v is not None for v in (s.value_dim, s.scale, s.chunk, s.sinks, s.q_norm, s.k_norm, s.head_gate, s.q_bias,
-                                                                 s.k_bias, s.v_bias, s.value_family, s.value_blend))
+                                                                 s.k_bias, s.v_bias, s.value_family, s.value_blend, getattr(s, "score_cap", None)))
                 or getattr(s, "qk_unit_rms", False) or getattr(s.position, "kind", None) in ("rotary_partial", "rotary_interleaved"))
 
     @classmethod
@@ -149,10 +155,11 @@ class Attention(Mixer):
         if spec.k_proj is not None:            # (a layer that reads another layer's pages has no keys and values of its own)
             needs += [TensorNeed(spec.k_proj, (kv, d)), TensorNeed(spec.v_proj, (spec.n_kv_heads * vd, d))]
         needs.append(TensorNeed(spec.o_proj, (d, spec.n_heads * vd)))
+        whole = getattr(spec, "qk_norm_whole", False)          # one norm over all heads of a projection, with a weight per channel of all heads
         if spec.q_norm is not None:
-            needs.append(TensorNeed(spec.q_norm, (spec.head_dim,), "norm"))
+            needs.append(TensorNeed(spec.q_norm, (a if whole else spec.head_dim,), "norm"))
         if spec.k_norm is not None and spec.k_proj is not None:
-            needs.append(TensorNeed(spec.k_norm, (spec.head_dim,), "norm"))
+            needs.append(TensorNeed(spec.k_norm, (kv if whole else spec.head_dim,), "norm"))
         if spec.sinks is not None:
             needs.append(TensorNeed(spec.sinks, (spec.n_heads,)))
         if spec.head_gate is not None:
@@ -213,10 +220,10 @@ class Attention(Mixer):
         ops.norm_rope_store(q, k, v, self.q_norm, self.k_norm if k is not None else None, s.qk_norm_eps, cos, sin, turned, ctx.row_pos, ctx.row_slot,
                             cache.table, q_ready, cache.kv, cache.page_size, s.n_heads, s.n_kv_heads, s.head_dim, vd,
                             biases=biases if any(b is not None for b in biases) else None, blend=blend, keep=keep, neighbours=neighbours,
-                            unit_rms=self.unit_rms, norm_last=self.unit_rms, v_scale=self.out_scale)
+                            unit_rms=self.unit_rms, norm_last=self.unit_rms, v_scale=self.out_scale, norm_all=self.norm_whole)
         att = torch.empty((T, s.n_heads * vd), dtype=cache.kv.dtype, device=ctx.device)
         return ops.attention_general(q_ready, cache.kv, att, ctx, cache.table, s.n_heads, s.n_kv_heads, s.head_dim, page_size=cache.page_size,
-                                     value_dim=vd, window=s.window, chunk=s.chunk, scale=s.scale, sinks=self.sinks, gate=gate)
+                                     value_dim=vd, window=s.window, chunk=s.chunk, scale=s.scale, sinks=self.sinks, gate=gate, cap=self.score_cap)
 
     out_scale = 1.0
 

@@ -34,6 +34,12 @@ class RoutedExperts(FeedForward):
         if s.n_experts > ops.ROUTER_MAX_EXPERTS or s.top > ops.ROUTER_MAX_TOP:
             raise ValueError(f"routed experts: at most {ops.ROUTER_MAX_EXPERTS} experts and {ops.ROUTER_MAX_TOP} a row")
         self.router = tensors[s.router]
+        self.limit = float(getattr(s, "activation_limit", 0.0))
+        self.groups = (s.n_groups, s.groups_kept) if getattr(s, "n_groups", 1) > 1 else None
+        self.floor = float(getattr(s, "renormalize_floor", 0.0))
+        # the shared feed-forward's gate is one more row of the router's matrix: its logit comes out of the router's product, in 32-bit
+        self.shared_gated = getattr(s, "shared_gate", None) is not None
+        self.router_all = torch.cat([self.router, tensors[s.shared_gate].reshape(1, -1)], dim=0).contiguous() if self.shared_gated else self.router
         self.w_down = torch.stack([tensors[n] for n in s.down_projs]).contiguous()
         if self.w_down.dtype == torch.bfloat16 and dtype == torch.bfloat16 and s.intermediate_size % ops.EXPERT_ROW_GROUP == 0:
             # gates and up products in one stack, as the product with the gate inside reads them
@@ -57,23 +63,36 @@ class RoutedExperts(FeedForward):
             needs += [TensorNeed(g, (i, d)), TensorNeed(u, (i, d)), TensorNeed(w, (d, i))]
         if s.shared is not None:
             needs += feed_forward_class(s.shared).tensor_needs(s.shared)
+        if getattr(s, "shared_gate", None) is not None:
+            needs.append(TensorNeed(s.shared_gate, (1, d)))
         return needs
 
     def weights_read_per_step(self):
         """What a step of few rows reads: the router, `top` experts a row at most (here: of one row), the shared feed-forward."""
         s = self.spec
         share = [w[:min(s.top, s.n_experts)] for w in (self.w_gate, self.w_up, self.w_down) if w is not None]
-        return [self.router, *share] + ([self.shared] if self.shared is not None else [])
+        return [self.router_all, *share] + ([self.shared] if self.shared is not None else [])
 
     def forward(self, h, residual, ctx, then=None, overwrite=False):
         s, T, dev = self.spec, ctx.n_rows, ctx.device
         rows = h.materialize() if isinstance(h, NormedRows) else h
         ids = torch.empty((T, s.top), dtype=torch.int32, device=dev)
         weights = torch.empty((T, s.top), dtype=torch.float32, device=dev)
-        ops.route_rows(rows, self.router, s.top, ids, weights, s.score, s.renormalize)
-        ops.routed_experts(rows, self.w_gate, self.w_up, self.w_down, ids, weights, residual, accumulate=not overwrite, weigh=s.weigh, activation=s.activation)
-        if self.shared is not None:
+        ops.route_rows(rows, self.router, s.top, ids, weights, s.score, s.renormalize, groups=self.groups, floor=self.floor)
+        ops.routed_experts(rows, self.w_gate, self.w_up, self.w_down, ids, weights, residual, accumulate=not overwrite, weigh=s.weigh, activation=s.activation,
+                           limit=self.limit)
+        if self.shared is not None and not self.shared_gated:
             self.shared.forward(rows, residual, ctx)
+        elif self.shared is not None:          # its result in rows of its own, added times the row's gate
+            gate = torch.empty((T, 1), dtype=torch.float32, device=dev)
+            ops.gemm_exact(rows, self.router_all[s.n_experts:], gate)
+            if getattr(self.shared, "can_overwrite", False):
+                y = torch.empty_like(residual)
+                self.shared.forward(rows, y, ctx, overwrite=True)
+            else:
+                y = torch.zeros_like(residual)
+                self.shared.forward(rows, y, ctx)
+            ops.add_rows_gated(residual, y, gate)
         return None
 
 

@@ -68,7 +68,11 @@ class LatentAttention(Mixer):
             self.position = position_class(s.position)(s.position, tensors, dtype, device)
             if not hasattr(self.position, "pair_tables") or s.position.rotary_dim != s.rotary_dim:
                 raise ValueError("latent attention: the position encoding must give angles for rotary_dim / 2 neighbouring pairs")
-        self.w_down = _pad_rows(torch.cat([tensors[s.dq_proj], tensors[s.dkv_proj]], dim=0).contiguous())
+        # one product for both latents and, where every head's output has a gate, the gates' logits behind them
+        self.gate_at = s.q_rank + s.kv_rank + s.rotary_dim
+        gates = [tensors[s.head_gate]] if getattr(s, "head_gate", None) is not None else []
+        self.gated = bool(gates)
+        self.w_down = _pad_rows(torch.cat([tensors[s.dq_proj], tensors[s.dkv_proj], *gates], dim=0).contiguous())
         self.q_norm, self.kv_norm = tensors[s.dq_norm], tensors[s.dkv_norm]
         self.w_uq = tensors[s.uq_proj]
         # per head: W_uk_h^T [kv_rank, head_dim] (folded into the queries) and W_uv_h [value_dim, kv_rank] (applied to the attended latent)
@@ -98,7 +102,7 @@ class LatentAttention(Mixer):
         return [TensorNeed(s.dq_proj, (s.q_rank, d)), TensorNeed(s.dq_norm, (s.q_rank,), "norm"), TensorNeed(s.uq_proj, (s.n_heads * (s.head_dim + s.rotary_dim), s.q_rank)),
                 TensorNeed(s.dkv_proj, (s.kv_rank + s.rotary_dim, d)), TensorNeed(s.dkv_norm, (s.kv_rank,), "norm"),
                 TensorNeed(s.uk_proj, (s.n_heads * s.head_dim, s.kv_rank)), TensorNeed(s.uv_proj, (s.n_heads * s.value_dim, s.kv_rank)),
-                TensorNeed(s.o_proj, (d, s.n_heads * s.value_dim))]
+                TensorNeed(s.o_proj, (d, s.n_heads * s.value_dim))] + ([TensorNeed(s.head_gate, (s.n_heads, d))] if getattr(s, "head_gate", None) is not None else [])
 
     @classmethod
     def cache_need(cls, spec):
@@ -131,6 +135,8 @@ class LatentAttention(Mixer):
             attended = attended.to(activation_dtype_for(self.w_uv, self.dtype))
         att = torch.empty((T, H * s.value_dim), dtype=self.att_dtype, device=dev)
         heads_product(attended, self.w_uv, att, H)
+        if self.gated:
+            ops.head_gate(att, down[:, self.gate_at:self.gate_at + H], H, s.value_dim)
         if overwrite:
             linear(att, self.w_o, residual)
             return None

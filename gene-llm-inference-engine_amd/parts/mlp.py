@@ -27,8 +27,9 @@ class SwiGlu(FeedForward):
         self.activation = getattr(spec, "activation", "silu")
         if self.activation not in ops.ACTIVATIONS:
             raise ValueError(f"feed-forward: unknown activation {self.activation!r}; known: {', '.join(ops.ACTIVATIONS)}")
+        self.limit = float(getattr(spec, "activation_limit", 0.0))
         self.fused = (self.in_dtype == torch.bfloat16 and self.mid_dtype == torch.bfloat16 and up.dtype == torch.bfloat16
-                      and spec.intermediate_size % 16 == 0 and spec.hidden_size % 8 == 0)
+                      and spec.intermediate_size % 16 == 0 and spec.hidden_size % 8 == 0 and self.activation in ops.FUSED_GATE_ACTIVATIONS)
         self.w_gate_up = ops.interleave_gate_up(gate, up) if self.fused else torch.cat([gate, up], dim=0).contiguous()
 
     @classmethod
@@ -48,7 +49,7 @@ class SwiGlu(FeedForward):
             gate_up = torch.empty((T, 2 * inter), dtype=torch.float32, device=ctx.device)
             linear(h, self.w_gate_up, gate_up)
             mid = torch.empty((T, inter), dtype=self.mid_dtype, device=ctx.device)
-            ops.act_mul(gate_up, mid, self.activation)
+            ops.act_mul(gate_up, mid, self.activation, self.limit)
         if overwrite:
             linear(mid, self.w_down, residual)
             return None

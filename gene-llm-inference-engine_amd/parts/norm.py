@@ -1,5 +1,5 @@
 """RMS norm: out = w * (x * rsqrt(mean(x^2) + eps)), eps inside the root, the weight as stored
-(reference: src/kernels/kernels.cpp:72-83).
+(reference: src/kernels/kernels.cpp:72-83), or, where the spec says so, the stored weight plus a constant.
 
 A norm may be handed on *unapplied* (`deferred`): `NormedRows` names the rows (optionally a
 selection of them), the weight and eps; whoever consumes it asks for the rows (`materialize`), and
@@ -67,6 +67,8 @@ class RmsNorm(Norm):
     def __init__(self, spec, tensors, dtype, device):
         super().__init__(spec, tensors, dtype, device)
         self.weight = tensors[spec.weight]
+        if getattr(spec, "weight_offset", 0.0):          # weights stored around zero: the sum is made once, in 32-bit (bfloat16 would lose the stored part's digits)
+            self.weight = (self.weight.float() + float(spec.weight_offset)).contiguous()
         self.eps = float(spec.eps)
         # the weights once more in 32-bit, for a product that applies them to rows it has just written (`handed_weight`); made
         # here, not at first use, which might fall into the capture of a graph
