@@ -4,6 +4,7 @@
     python bench.py --fekorax [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]     (another record: see `fekorax_beside_llama`)
     python bench.py --rigalorn [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]    (another record: see `rigalorn_beside_fekorax`)
     python bench.py --zidevik [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]     (another record: see `zidevik_beside_rigalorn`)
+    python bench.py --mimitar [--sizes 1b,8b] [--layers L] [--batch B] [--prefill-tokens T]     (another record: see `mimitar_beside_zidevik`)
 
 A step is one decode step of the whole batch (default batch 8, each request on a 2,048-token
 prompt in a 4,096-token context), through the scheduler with its defaults.  After W warm-up steps,
@@ -217,6 +218,58 @@ def zidevik_beside_rigalorn(args) -> int:
     return 0
 
 
+def mimitar_beside_zidevik(args) -> int:
+    """The Mimitar design at layer shapes of real models beside the Zidevik design (the nearest the engine has: attention with a scale
+    of its own and a rotation of a part of the head, routed experts with a shared one), the Rigalorn design (attention through
+    latents) and the Llama decoder at the same shapes, random weights; measured as `fekorax_beside_llama` measures.  A Mimitar model
+    of L layers here carries 4 copies of the residual stream; its layers take turns of four: attention with the Llama layer's heads
+    (a norm over the whole query and key projections, a rotation of half of each head with stretched frequencies, scores capped at
+    30) and the Llama layer's feed-forward with clamped halves; the same attention with 8 experts of a quarter of that inner size
+    in 4 groups of which 2 are kept, 2 experts a token, and a gated shared expert of half of it; the first layer once more with its
+    own cache (no weights of its own); attention through latents (Rigalorn's sizes, a gate per head) with the experts.  Every
+    mixer's input is blended with the token before.  One JSON line."""
+    import torch
+    T, batch, L, steps = args.prefill_tokens, args.batch, args.layers or 8, args.steps
+    gen = torch.Generator().manual_seed(1)
+    record = {"metric": "Mimitar beside Zidevik, Rigalorn and Llama at equal layer shapes: prefill tok/s, decode ms a step, ms by kernel", "dtype": args.dtype, "layers": L,
+              "prefill_tokens": T, "decode_batch": batch, "data": "synthetic: random weights by formula, uniform random token ids", "sizes": {}}
+    for size in args.sizes.split(","):
+        D, H, G, hd, ff, vocab = FEKORAX_SIZES[size]
+        mlp = dict(kind="dense", ff=ff)
+        llama = dict(architectures=["LlamaForCausalLM"], hidden_size=D, intermediate_size=ff, num_hidden_layers=L, num_attention_heads=H,
+                     num_key_value_heads=G, head_dim=hd, vocab_size=vocab, max_position_embeddings=T + 1024, rope_theta=500000.0, rms_norm_eps=1e-5,
+                     tie_word_embeddings=True)
+        delta = dict(type="delta", mlp=mlp, mixer=dict(heads=max(1, H // 4), kv_heads=max(1, H // 8), dim=hd, vdim=2 * hd, conv=4))
+        latent = dict(type="latent_attention", mlp=mlp, mixer=dict(heads=H, dim=hd, rot_dim=hd // 2, vdim=hd, q_rank=12 * hd, kv_rank=4 * hd, scale=(1.5 * hd) ** -0.5,
+                                                                    rot=dict(dims=hd // 2, base=500000.0), mask=dict(size=1024)))
+        blended = dict(type="attention", mlp=mlp, mixer=dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, v_mix=True, mask=dict(size=1024), rot=dict(
+            dims=hd // 2, base=10000.0, scaling=dict(factor=4.0, original=4096, fast=16.0, slow=2.0))))
+        rigalorn = dict(architecture="Rigalorn", vocab=vocab, width=D, embedding=dict(scale=D ** 0.5), norm=dict(eps=1e-5), max_positions=T + 1024,
+                        layers=([delta, latent, blended, delta] * ((L + 3) // 4))[:L])
+        mixer = dict(left=dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, rot=dict(dims=hd // 2, base=500000.0)), left_scale=1.0,
+                     right=dict(inner=2 * D, state=16, dt_rank=D // 16, conv=4), right_scale=1.0)
+        moe = dict(kind="moe", router=dict(experts=8, top=2), expert=dict(ff=ff // 4), shared=dict(ff=ff // 2))
+        zidevik = dict(architecture="Zidevik", vocab=vocab, width=D, norm=dict(eps=1e-5), max_positions=T + 1024, logit_softcap=30.0, token_side=dict(dim=256),
+                       loop=dict(start=0, stop=min(2, L), times=2), layers=[dict(type="parallel", mixer=mixer, mlp=mlp if i % 2 == 0 else moe) for i in range(L)])
+        m_dense = dict(kind="dense", ff=ff, limit=7.0)
+        m_moe = dict(kind="moe", router=dict(experts=8, top=2, groups=dict(count=4, keep=2)), expert=dict(ff=ff // 4, limit=7.0), shared=dict(ff=ff // 2, limit=7.0))
+        m_att = dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, softcap=30.0,
+                     rot=dict(dims=hd // 2, base=500000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+        m_latent = dict(heads=H, dim=hd, rot_dim=hd // 2, vdim=hd, q_rank=12 * hd, kv_rank=4 * hd, scale=(1.5 * hd) ** -0.5,
+                        rot=dict(dims=hd // 2, base=500000.0, scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0)))
+        four = lambda i: [dict(type="attention", mixer=m_att, mlp=m_dense), dict(type="attention", mixer=m_att, mlp=m_moe),
+                          dict(type="attention", mixer=m_att, mlp=m_dense, weights_of=i), dict(type="latent_attention", mixer=m_latent, mlp=m_moe)]
+        mimitar = dict(architecture="Mimitar", vocab=vocab, width=D, norm=dict(eps=1e-5), streams=4, residual_mult=0.7, logit_scale=0.5, max_positions=T + 1024,
+                       layers=[l for i in range(0, L, 4) for l in four(i)][:L])
+        record["sizes"][size] = {}
+        for name, cfg in (("llama", llama), ("rigalorn", rigalorn), ("zidevik", zidevik), ("mimitar", mimitar)):
+            if args.only and name not in args.only.split(","):
+                continue
+            record["sizes"][size][name] = _measure_design(cfg, args, T, batch, steps, vocab, gen)
+    print(json.dumps(record))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -231,8 +284,9 @@ def main() -> int:
     ap.add_argument("--fekorax", action="store_true", help="another measurement: the Fekorax design beside Llama at equal layer shapes (see fekorax_beside_llama)")
     ap.add_argument("--rigalorn", action="store_true", help="another measurement: the Rigalorn design beside Fekorax and Llama at equal layer shapes (see rigalorn_beside_fekorax)")
     ap.add_argument("--zidevik", action="store_true", help="another measurement: the Zidevik design beside Rigalorn and Llama at equal layer shapes (see zidevik_beside_rigalorn)")
-    ap.add_argument("--only", default="", help="with --rigalorn or --zidevik: the designs to measure, of llama, fekorax, rigalorn, zidevik (default: all)")
-    ap.add_argument("--sizes", default="1b,8b", help="with --fekorax, --rigalorn or --zidevik: layer shapes, of " + ", ".join(FEKORAX_SIZES))
+    ap.add_argument("--mimitar", action="store_true", help="another measurement: the Mimitar design beside Zidevik, Rigalorn and Llama at equal layer shapes (see mimitar_beside_zidevik)")
+    ap.add_argument("--only", default="", help="with --rigalorn, --zidevik or --mimitar: the designs to measure, of llama, fekorax, rigalorn, zidevik, mimitar (default: all)")
+    ap.add_argument("--sizes", default="1b,8b", help="with --fekorax, --rigalorn, --zidevik or --mimitar: layer shapes, of " + ", ".join(FEKORAX_SIZES))
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine")
@@ -244,6 +298,8 @@ def main() -> int:
         return rigalorn_beside_fekorax(args)
     if args.zidevik:
         return zidevik_beside_rigalorn(args)
+    if args.mimitar:
+        return mimitar_beside_zidevik(args)
 
     import torch
     from geneinfer_amd.config import LlamaConfig

@@ -31,11 +31,22 @@ __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_ex
 //   sinks   [n_heads]: exp(sinks[h]) joins the softmax's denominator of head h (a score without a key or a value), once a row:
 //           where a row's keys are shared out over splits or waves, the first of them counts it;
 //   gate    [rows, gate_stride]: head h's output of row t is multiplied by sigmoid(gate[t * gate_stride + h]).
+//   cap     > 0: a scaled score s becomes cap * tanh(s / cap) before the softmax.
 struct Extras {
     int chunk;
     const float* sinks;
     const float* gate;
     long gate_stride;
+    float cap;
+};
+// Capped scores, in units of log2 e: with a cap the kernels take scale2 = 1 and turn every product s into
+// cap log2(e) tanh(s scale / cap) first; tanh(x) = 1 - 2 / (1 + e^(2x)), the exponential as one exp2 (it may overflow: the
+// reciprocal of infinity is 0 and the result 1).
+struct ScoreCap {
+    float twice_inv2, cap2;          // 2 log2(e) scale / cap, cap log2(e); cap2 = 0: no cap
+    __device__ __forceinline__ ScoreCap(float scale, float cap) : twice_inv2(cap > 0.f ? 2.f * LOG2E * scale / cap : 0.f), cap2(cap > 0.f ? cap * LOG2E : 0.f) {}
+    __device__ __forceinline__ bool on() const { return cap2 > 0.f; }
+    __device__ __forceinline__ float of(float s) const { return cap2 * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + exp2_fast(s * twice_inv2))); }
 };
 // The first position a row at `p` sees.
 __device__ __forceinline__ int lowest_seen(int p, int window, int chunk) {
@@ -78,7 +89,7 @@ constexpr int KV_TILE = 64;
 // true maximum some row of 32 has a new one in most tiles.  The first keys a row sees always set it (-inf + slack = -inf).
 constexpr float MAX_SLACK = 8.0f;
 
-template <int HD, int NW, int PAIR>
+template <int HD, int NW, int PAIR, bool CAP>
 __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
                                                                           bf16_t* __restrict__ out, const int4* __restrict__ tiles,
                                                                           const int* __restrict__ table, int table_stride, long page_stride,
@@ -122,7 +133,8 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
     const int wave_first = wave_full ? pos0 + wv * 32 : -1;             // keys up to here are seen by every row of the wave (none if rows are missing)
     const int wave_lo_max = lowest_seen(wave_last, window, extra.chunk);      // ... and keys from here on
     const int wave_lo_min = lowest_seen(pos0 + wv * 32, window, extra.chunk); // no row of the wave sees a key before this one
-    const float scale2 = scale * LOG2E;
+    const ScoreCap capped(scale, CAP ? extra.cap : 0.f);          // (a kernel of its own where scores are capped: the others are as they were)
+    const float scale2 = CAP ? 1.0f : scale * LOG2E;
 
     bf16x8 qreg[QSTEPS];
 #pragma unroll
@@ -256,6 +268,10 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
             }
             // element v of s: key position kv_base + 8*(v/4) + 4*hf + v%4, query row `col`.  Scores are kept
             // in units of log2 e (scale2 = scale * log2 e), so that e^(s - m) is one exp2.
+            if constexpr (CAP) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[v] = capped.of(s[v]);
+            }
             const bool inside = kv_base + 31 <= wave_first && kv_base >= wave_lo_max;     // every key here is seen by every row of the wave
             float mx = -INFINITY;
             if (inside) {
@@ -382,7 +398,7 @@ __global__ __launch_bounds__(128 * NW * PAIR) void attention_prompt_kernel(const
 // The rows of a key tile are taken in another order by the score product: row i of the matrix instruction reads key
 // pi(i) = 16 (i / 16) + 8 ((i / 4) % 2) + 4 ((i / 8) % 2) + i % 4 of its 32, so that the 8 scores a lane holds for the
 // next product's k index are 8 consecutive keys, and the value operand is one 16-byte read (8 positions of a channel).
-template <int HD, int NW>
+template <int HD, int NW, bool CAP>
 __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_wide_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ cache,
                                                                        bf16_t* __restrict__ out, const int4* __restrict__ tiles,
                                                                        const int* __restrict__ table, int table_stride, long page_stride,
@@ -422,7 +438,8 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
     const int wave_first = wave_full ? pos0 + wv * 32 : -1;
     const int wave_lo_max = lowest_seen(wave_last, window, extra.chunk);
     const int wave_lo_min = lowest_seen(pos0 + wv * 32, window, extra.chunk);
-    const float scale2 = scale * LOG2E;
+    const ScoreCap capped(scale, CAP ? extra.cap : 0.f);          // (a kernel of its own where scores are capped: the others are as they were)
+    const float scale2 = CAP ? 1.0f : scale * LOG2E;
 
     bf16x8 qreg[QSTEPS];
 #pragma unroll
@@ -523,6 +540,12 @@ __global__ __launch_bounds__(64 * NW, HD == 128 ? 2 : 3) void attention_prompt_w
             }
             // element v of s[h]: key kv0 + 32 h + 16 (v / 8) + 8 hf + v % 8, query row `col`; in units of log2 e after scale2
             // (keys some row of the wave does not see are masked where they stand, before the part that every tile walks)
+            if constexpr (CAP) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[h][v] = capped.of(s[h][v]);
+            }
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int kv_base = kv0 + 32 * h;
@@ -665,7 +688,7 @@ __device__ __forceinline__ uint4 rotated8(const Pairs8& p, const Angles8& u) {
     return uint4{w[0], w[1], w[2], w[3]};
 }
 
-template <int HD, bool FUSED>
+template <int HD, bool FUSED, bool CAP>
 __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_decode_kernel(
     const bf16_t* __restrict__ q, const float* __restrict__ qf, const float* __restrict__ kf, const float* __restrict__ vf, long ldq, long ldk,
     long ldv, const float* __restrict__ cos_t, const float* __restrict__ sin_t, bf16_t* __restrict__ cache, float* __restrict__ part,
@@ -709,7 +732,8 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
     const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
     auto page_index = [&](int kv) { return page_shift >= 0 ? kv >> page_shift : kv / page_size; };
     auto place_of = [&](int kv) { return page_shift >= 0 ? kv & (page_size - 1) : kv % page_size; };
-    const float scale2 = scale * LOG2E;            // scores are kept in units of log2 e: e^(s - m) is one exp2
+    const ScoreCap capped(scale, CAP ? extra.cap : 0.f);
+    const float scale2 = CAP ? 1.0f : scale * LOG2E;            // scores are kept in units of log2 e: e^(s - m) is one exp2
     const long v_plane = (long)n_kv * page_size * HD;
     const bf16_t* kbase = cache + (long)g * page_size * HD;
     const bf16_t* vbase = cache + v_plane + (long)g * HD * page_size;
@@ -846,6 +870,12 @@ __global__ __launch_bounds__(64 * DecodeShape<HD>::MAX_WAVES) void attention_dec
             for (int ks = 0; ks < KSTEPS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(k_use[t][ks]), qreg[ks], s[t], 0, 0, 0);
         }
         // element v of s[t]: key position kv0 + 16*t + 4*q4 + v, query head r
+        if constexpr (CAP) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) s[t][v] = capped.of(s[t][v]);
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -1018,9 +1048,9 @@ GI_API int gi_attention_bf16_supports(int hd, int page_size, int prompt) {
 GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out, const int* tiles, int n_tiles, int rows_per_tile, int paired,
                                     const int* table, int table_stride, long page_stride, int page_size, int n_heads, int n_kv, int hd,
                                     int window, float scale, int n_splits, const int* tile_first, const int* rows, int n_rows, float* part,
-                                    long part_floats, int chunk, const float* sinks, const float* gate, long gate_stride, hipStream_t stream) {
-    GI_REQUIRE(chunk >= 0 && (gate == nullptr || gate_stride >= n_heads), "attention_prompt: bad chunk or gate stride");
-    const Extras extra = {chunk, sinks, gate, gate_stride};
+                                    long part_floats, int chunk, const float* sinks, const float* gate, long gate_stride, float cap, hipStream_t stream) {
+    GI_REQUIRE(chunk >= 0 && cap >= 0.f && (gate == nullptr || gate_stride >= n_heads), "attention_prompt: bad chunk, cap or gate stride");
+    const Extras extra = {chunk, sinks, gate, gate_stride, cap};
     GI_REQUIRE(rows_per_tile == 64 || rows_per_tile == 128, "attention_prompt: tiles of %d rows are not supported (64 or 128)", rows_per_tile);
     GI_REQUIRE(n_tiles > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_prompt: bad counts (%d tiles, %d heads, %d kv heads)",
                n_tiles, n_heads, n_kv);
@@ -1042,9 +1072,16 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
         GI_REQUIRE((long)n_tiles * n_splits <= 65535, "attention_prompt: %d tiles in %d splits are too many for one launch", n_tiles, n_splits);
         dim3 wgrid(n_heads, n_tiles * n_splits);
 #define WIDE(HD, NW)                                                                                                                    \
-    attention_prompt_wide_kernel<HD, NW><<<wgrid, 64 * NW, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
-                                                                       table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, \
-                                                                       tile_first, part, paired ? 1 : 0, extra)
+    do {                                                                                                                                \
+        if (extra.cap > 0.f)                                                                                                            \
+            attention_prompt_wide_kernel<HD, NW, true><<<wgrid, 64 * NW, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
+                                                                                     table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, \
+                                                                                     tile_first, part, paired ? 1 : 0, extra);            \
+        else                                                                                                                            \
+            attention_prompt_wide_kernel<HD, NW, false><<<wgrid, 64 * NW, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, table, \
+                                                                                      table_stride, page_stride, page_size, n_heads, n_kv, window, scale, n_splits, \
+                                                                                      tile_first, part, paired ? 1 : 0, extra);           \
+    } while (0)
         if (hd == 64) { if (rows_per_tile == 64) WIDE(64, 2); else WIDE(64, 4); }
         else WIDE(128, 4);      // (tiles of 64 rows too: two of its waves then only load; a workgroup of two waves would need 16 loads a wave and more registers than two to a SIMD leave)
 #undef WIDE
@@ -1059,9 +1096,16 @@ GI_API int gi_attention_prompt_bf16(const void* q, const void* cache, void* out,
     const bool pairs = paired && hd <= 64;
     dim3 grid((pairs ? n_tiles / 2 : n_tiles) * n_splits, n_heads);
 #define GO_(HD, NW, PAIR)                                                                                                               \
-    attention_prompt_kernel<HD, NW, PAIR><<<grid, 128 * NW * PAIR, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, \
-                                                                                table, table_stride, page_stride, page_size, n_heads, n_kv, window, \
-                                                                                scale, n_splits, tile_first, part, extra)
+    do {                                                                                                                                \
+        if (extra.cap > 0.f)                                                                                                            \
+            attention_prompt_kernel<HD, NW, PAIR, true><<<grid, 128 * NW * PAIR, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, \
+                                                                                              table, table_stride, page_stride, page_size, n_heads, n_kv, window, \
+                                                                                              scale, n_splits, tile_first, part, extra);  \
+        else                                                                                                                            \
+            attention_prompt_kernel<HD, NW, PAIR, false><<<grid, 128 * NW * PAIR, 0, stream>>>((const bf16_t*)q, (const bf16_t*)cache, (bf16_t*)out, (const int4*)tiles, \
+                                                                                               table, table_stride, page_stride, page_size, n_heads, n_kv, window, \
+                                                                                               scale, n_splits, tile_first, part, extra); \
+    } while (0)
 #define GO(HD)                                                                                                                          \
     do {                                                                                                                                \
         if (rows_per_tile == 64) { if (pairs) GO_(HD, 2, (HD <= 64 ? 2 : 1)); else GO_(HD, 2, 1); }                                     \
@@ -1100,7 +1144,7 @@ GI_API int gi_attention_decode_workgroups_per_unit(int hd, int fused, int n_wave
     const size_t lds = decode_lds_bytes(hd, n_waves, gh);
     int n = 0;
     hipError_t e = hipErrorInvalidValue;
-#define ASK2(HD, FUSED_) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)attention_decode_kernel<HD, FUSED_>, 64 * n_waves, lds)
+#define ASK2(HD, FUSED_) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void*)attention_decode_kernel<HD, FUSED_, false>, 64 * n_waves, lds)
 #define ASK(HD) do { if (fused) ASK2(HD, true); else ASK2(HD, false); } while (0)
     if (hd == 32) ASK(32); else if (hd == 64) ASK(64); else if (hd == 96) ASK(96); else if (hd == 128) ASK(128); else if (hd == 256) ASK(256);
 #undef ASK
@@ -1122,9 +1166,9 @@ GI_API int gi_attention_decode_bf16(const void* q, const float* qf, const float*
                                     const float* cos_t, const float* sin_t, void* cache, void* out, float* part, long part_floats,
                                     const int* rows, int n_rows, const int* pos, const int* slots, const int* table, int table_stride,
                                     long page_stride, int page_size, int n_heads, int n_kv, int hd, int window, float scale, int n_splits,
-                                    int n_waves, int chunk, const float* sinks, const float* gate, long gate_stride, hipStream_t stream) {
-    GI_REQUIRE(chunk >= 0 && (gate == nullptr || gate_stride >= n_heads), "attention_decode: bad chunk or gate stride");
-    const Extras extra = {chunk, sinks, gate, gate_stride};
+                                    int n_waves, int chunk, const float* sinks, const float* gate, long gate_stride, float cap, hipStream_t stream) {
+    GI_REQUIRE(chunk >= 0 && cap >= 0.f && (gate == nullptr || gate_stride >= n_heads), "attention_decode: bad chunk, cap or gate stride");
+    const Extras extra = {chunk, sinks, gate, gate_stride, cap};
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention_decode: bad counts (%d rows, %d heads, %d kv heads)",
                n_rows, n_heads, n_kv);
     GI_REQUIRE(gi_attention_bf16_supports(hd, page_size, 0), "attention_decode: head size %d with page size %d is not supported", hd, page_size);
@@ -1152,15 +1196,17 @@ GI_API int gi_attention_decode_bf16(const void* q, const float* qf, const float*
     GI_REQUIRE(lds <= 64 * 1024, "attention_decode: %d heads of size %d per key/value head do not fit", gh, hd);
     lds = decode_lds_bytes(hd, n_waves, gh);
     dim3 grid(n_rows, n_kv * hg, n_splits);
-#define GO2(HD, FUSED_)                                                                                                                    \
-    attention_decode_kernel<HD, FUSED_><<<grid, 64 * n_waves, lds, stream>>>((const bf16_t*)q, qf, kf, vf, ldq, ldk, ldv, cos_t, sin_t,   \
-                                                                             (bf16_t*)cache, part, (bf16_t*)out, rows, pos, slots, table, \
-                                                                             table_stride, page_stride, page_size, n_heads, n_kv, window,  \
-                                                                             scale, n_splits, gh, extra)
-#define GO(HD)                    \
-    do {                          \
-        if (qf) GO2(HD, true);    \
-        else GO2(HD, false);      \
+#define GO2(HD, FUSED_, CAP_)                                                                                                              \
+    attention_decode_kernel<HD, FUSED_, CAP_><<<grid, 64 * n_waves, lds, stream>>>((const bf16_t*)q, qf, kf, vf, ldq, ldk, ldv, cos_t, sin_t, \
+                                                                                   (bf16_t*)cache, part, (bf16_t*)out, rows, pos, slots, table, \
+                                                                                   table_stride, page_stride, page_size, n_heads, n_kv, window, \
+                                                                                   scale, n_splits, gh, extra)
+    GI_REQUIRE(!(qf && extra.cap > 0.f), "attention_decode: capped scores are not served from unrotated products");
+#define GO(HD)                                         \
+    do {                                               \
+        if (qf) GO2(HD, true, false);                  \
+        else if (extra.cap > 0.f) GO2(HD, false, true); \
+        else GO2(HD, false, false);                    \
     } while (0)
     if (hd == 32) GO(32); else if (hd == 64) GO(64); else if (hd == 96) GO(96); else if (hd == 128) GO(128); else GO(256);
 #undef GO

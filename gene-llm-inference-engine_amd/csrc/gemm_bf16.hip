@@ -34,9 +34,10 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2, EPI_GATED_BF16 = 3, EPI_QKV_ROPE = 4, EPI_GATED_GELU_BF16 = 5 };
-// The two gated epilogues differ in the activation alone: SiLU (EPI_GATED_BF16), or the tanh form of GELU.
-__host__ __device__ constexpr bool is_gated(int epi) { return epi == EPI_GATED_BF16 || epi == EPI_GATED_GELU_BF16; }
+enum Epilogue : int { EPI_STORE_F32 = 0, EPI_ADD_F32 = 1, EPI_STORE_BF16 = 2, EPI_GATED_BF16 = 3, EPI_QKV_ROPE = 4, EPI_GATED_GELU_BF16 = 5, EPI_GATED_CLAMP_BF16 = 6 };
+// The gated epilogues differ in the activation alone: SiLU (EPI_GATED_BF16), the tanh form of GELU, or the clamped form
+// g sigmoid(1.702 g) (u + 1) with g <- min(g, limit), u <- clamp(u, -limit, limit) (EPI_GATED_CLAMP_BF16; `limit` comes with `NormIn`).
+__host__ __device__ constexpr bool is_gated(int epi) { return epi == EPI_GATED_BF16 || epi == EPI_GATED_GELU_BF16 || epi == EPI_GATED_CLAMP_BF16; }
 
 __device__ __forceinline__ float silu_gate(float g, float u) { return (g * (1.0f / (1.0f + expf(-g)))) * u; }
 // The same with the hardware's exp2 and reciprocal (each within a unit or two in the last place of 32 bits): for results
@@ -52,10 +53,24 @@ __device__ __forceinline__ float gelu_gate_fast(float g, float u) {
     const float z = 0.7978845608028654f * (g + 0.044715f * g * g * g);
     return (g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -2.8853900817779268f))) * u;
 }
+__device__ __forceinline__ float clamp_gate(float g, float u, float limit) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * (1.0f / (1.0f + expf(-1.702f * g))) * (u + 1.0f);
+}
+__device__ __forceinline__ float clamp_gate_fast(float g, float u, float limit) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return (g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * (-1.702f * 1.4426950408889634f)))) * (u + 1.0f);
+}
 template <int EPI>
-__device__ __forceinline__ float gate_of(float g, float u) { return EPI == EPI_GATED_GELU_BF16 ? gelu_gate(g, u) : silu_gate(g, u); }
+__device__ __forceinline__ float gate_of(float g, float u, float limit) {
+    return EPI == EPI_GATED_CLAMP_BF16 ? clamp_gate(g, u, limit) : EPI == EPI_GATED_GELU_BF16 ? gelu_gate(g, u) : silu_gate(g, u);
+}
 template <int EPI>
-__device__ __forceinline__ float gate_fast_of(float g, float u) { return EPI == EPI_GATED_GELU_BF16 ? gelu_gate_fast(g, u) : silu_gate_fast(g, u); }
+__device__ __forceinline__ float gate_fast_of(float g, float u, float limit) {
+    return EPI == EPI_GATED_CLAMP_BF16 ? clamp_gate_fast(g, u, limit) : EPI == EPI_GATED_GELU_BF16 ? gelu_gate_fast(g, u) : silu_gate_fast(g, u);
+}
 
 __device__ __forceinline__ uint4 load16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
@@ -84,6 +99,7 @@ struct NormIn {                  // for a product whose rows A are g * x without
     int parts;
     float eps;
     int dim;                     // r = rsqrt(sum / dim + eps)
+    float limit;                 // of the clamped gated epilogue (nothing of the norm's: it travels here because every kernel takes this struct)
 };
 
 // Where an attention layer wants the sums of its q/k/v product (columns: n_heads * hd queries, n_kv * hd keys, n_kv * hd values):
@@ -243,7 +259,7 @@ constexpr int BN = 128, BK = 64, LDS_STRIDE = BK + 8;     // +8 bf16 (16 bytes) 
 
 template <int BM, int EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C,
-                                                             int M, int N, int K, long lda, long ldw, long ldc) {
+                                                             int M, int N, int K, long lda, long ldw, long ldc, float gate_limit) {
     constexpr int WM = BM / 2;                 // rows of a wave's tile (waves sit 2 x 2)
     constexpr int TM = WM / 32, TN = 2;        // 32x32 tiles per wave
     constexpr int A_CHUNKS = BM * BK / 8 / 256, W_CHUNKS = BN * BK / 8 / 256;   // 16-byte chunks per thread
@@ -321,7 +337,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled_kernel(const bf16_t* __re
                     // columns 32b .. 32b+15 are gates, 32b+16 .. 32b+31 the ups of outputs 16b .. 16b+15
                     const float up = __shfl_xor(acc[i][j][v], 16, 64);
                     if ((lane & 16) == 0 && m < M && n < N)
-                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(gate_of<EPI>(acc[i][j][v], up));
+                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(gate_of<EPI>(acc[i][j][v], up, gate_limit));
                 } else {
                     if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
                 }
@@ -501,7 +517,7 @@ __device__ __forceinline__ void piped_tile(const bf16_t* __restrict__ A, const b
                 if constexpr (is_gated(EPI)) {
                     const float up = __shfl_xor(acc[i][j][v], 16, 64);
                     if ((lane & 16) == 0 && m < M && n < N)
-                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(gate_of<EPI>(acc[i][j][v], up));
+                        ((bf16_t*)C)[(size_t)m * ldc + (n >> 5) * 16 + (lane & 15)] = f32_to_bf16(gate_of<EPI>(acc[i][j][v], up, norm_in.limit));
                 } else if constexpr (EPI != EPI_QKV_ROPE) {
                     if (m < M && n < N) write_out<EPI>(C, (size_t)m * ldc + n, acc[i][j][v]);
                 }
@@ -520,10 +536,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_bf16_piped_kernel
 // fill up a run's last tile hold anything; their results are stored like the others and nobody reads them.
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_bf16_grouped_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W, void* __restrict__ C, int M, int N,
-                                                               int K, long lda, long ldw, long ldc, const int* __restrict__ tile_group, long group_stride) {
+                                                               int K, long lda, long ldw, long ldc, const int* __restrict__ tile_group, long group_stride, float gate_limit) {
     const int g = tile_group[blockIdx.y];
     if (g < 0) return;
-    const NormIn no_norm_in = {nullptr, 0, 0.f, 1};
+    const NormIn no_norm_in = {nullptr, 0, 0.f, 1, gate_limit};
     const NormOut no_norm_out = {nullptr, nullptr, 0, nullptr};
     const RopeStore no_rope = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, 0};
     piped_tile<128, 128, 2, 2, 2, EPI>(A, W + (size_t)g * group_stride, C, M, N, K, lda, ldw, ldc, K, 0L, no_norm_in, no_rope, no_norm_out, blockIdx.y);
@@ -703,8 +719,8 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong_kernel(const bf16_t* _
 #pragma unroll
                     for (int q = 0; q < 2; ++q) {
                         const float rs = norm_in.squares != nullptr ? row_scale[wm + i * 32 + (lane & 31)] : 1.0f;
-                        const uint2 packed = {f32x2_to_bf16x2(gate_fast_of<EPI>(acc[i][j][4 * q] * rs, acc[i][j][4 * q + 8] * rs), gate_fast_of<EPI>(acc[i][j][4 * q + 1] * rs, acc[i][j][4 * q + 9] * rs)),
-                                              f32x2_to_bf16x2(gate_fast_of<EPI>(acc[i][j][4 * q + 2] * rs, acc[i][j][4 * q + 10] * rs), gate_fast_of<EPI>(acc[i][j][4 * q + 3] * rs, acc[i][j][4 * q + 11] * rs))};
+                        const uint2 packed = {f32x2_to_bf16x2(gate_fast_of<EPI>(acc[i][j][4 * q] * rs, acc[i][j][4 * q + 8] * rs, norm_in.limit), gate_fast_of<EPI>(acc[i][j][4 * q + 1] * rs, acc[i][j][4 * q + 9] * rs, norm_in.limit)),
+                                              f32x2_to_bf16x2(gate_fast_of<EPI>(acc[i][j][4 * q + 2] * rs, acc[i][j][4 * q + 10] * rs, norm_in.limit), gate_fast_of<EPI>(acc[i][j][4 * q + 3] * rs, acc[i][j][4 * q + 11] * rs, norm_in.limit))};
                         *reinterpret_cast<uint2*>(mine + (i * 32 + (lane & 31)) * STAGE_ROW + (jj * 16 + 8 * q + 4 * (lane >> 5)) * 2) = packed;
                     }
                 }
@@ -954,7 +970,7 @@ __global__ __launch_bounds__(512, MT == 2 ? 4 : 2) void gemm_bf16_skinny_kernel(
                 for (int v = 0; v < 4; ++v) {
                     const int m = t * 16 + 4 * q + v;
                     const float rs = scaled_rows ? row_scale[m] : 1.0f;
-                    if (m < M) ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 32 + (strip >> 1) * 16 + r] = f32_to_bf16(gate_of<EPI>(acc[t][v] * rs, other[strip + 1][t][lane][v] * rs));
+                    if (m < M) ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 32 + (strip >> 1) * 16 + r] = f32_to_bf16(gate_of<EPI>(acc[t][v] * rs, other[strip + 1][t][lane][v] * rs, norm_in.limit));
                 }
         }
     } else if (half == 0 && n < N) {
@@ -1055,7 +1071,7 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
 
 // The same for the gated product: columns 32b .. 32b+15 of the partial sums are gates, 32b+16 .. 32b+31 the ups of
 // outputs 16b .. 16b+15; the output [M, N/2] is silu(gate) * up in bfloat16.
-__global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* __restrict__ C, int M, int N, int splits, long ldc, int gelu) {
+__global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* __restrict__ C, int M, int N, int splits, long ldc, int epi, float limit) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int half = N / 2;
     if (i >= (size_t)M * half) return;
@@ -1066,7 +1082,7 @@ __global__ void skinny_reduce_gated_kernel(const float* __restrict__ P, bf16_t* 
         gate += P[((size_t)sp * M + m) * N + col];
         up += P[((size_t)sp * M + m) * N + col + 16];
     }
-    C[m * ldc + c] = f32_to_bf16(gelu ? gelu_gate(gate, up) : silu_gate(gate, up));
+    C[m * ldc + c] = f32_to_bf16(epi == EPI_GATED_CLAMP_BF16 ? clamp_gate(gate, up, limit) : epi == EPI_GATED_GELU_BF16 ? gelu_gate(gate, up) : silu_gate(gate, up));
 }
 
 // The same for the q/k/v product of an attention layer, N = (n_heads + 2 n_kv) * hd columns: the sums of a row are its queries,
@@ -1295,7 +1311,7 @@ __global__ __launch_bounds__(512, 4) void gemm_bf16_slim_kernel(const bf16_t* __
                     up += red[s * STRIPS + 1][0][src_lane][v];
                 }
                 if constexpr (HAND) { gate *= r; up *= r; }
-                ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 16 + c] = f32_to_bf16(gate_of<EPI>(gate, up));
+                ((bf16_t*)C)[(size_t)m * ldc + blockIdx.x * 16 + c] = f32_to_bf16(gate_of<EPI>(gate, up, norm_in.limit));
             } else {
                 float sum = 0.f;
 #pragma unroll
@@ -1492,14 +1508,14 @@ static int consumer_max_parts(int M) { return M <= 16 ? slim_max_parts(M) : M <=
 // 47.4 against 52.8.)
 static bool takes_pingpong(int M, int N) { return (long)((M + 255) / 256) * ((N + 255) / 256) >= gi_compute_units() * 3 / 4; }
 
-static const NormIn NO_NORM_IN = {nullptr, 0, 0.f, 1};
+static const NormIn NO_NORM_IN = {nullptr, 0, 0.f, 1, 0.f};
 static const NormOut NO_NORM_OUT = {nullptr, nullptr, 0, nullptr};
 
 static int reduce_partials(const float* scratch, void* C, int epi, int M, int N, int splits, long ldc, hipStream_t stream, NormIn norm_in = NO_NORM_IN,
                            NormOut norm_out = NO_NORM_OUT) {
     if (is_gated(epi)) {
         GI_REQUIRE(norm_in.squares == nullptr, "gemm_bf16: a gated product whose k is shared out cannot finish a norm handed on");
-        skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc, epi == EPI_GATED_GELU_BF16 ? 1 : 0);
+        skinny_reduce_gated_kernel<<<(unsigned)(((size_t)M * (N / 2) + 255) / 256), 256, 0, stream>>>(scratch, (bf16_t*)C, M, N, splits, ldc, epi, norm_in.limit);
     } else {
 #define REDUCE(VEC_)                                                                                                                    \
     do {                                                                                                                                \
@@ -1576,7 +1592,7 @@ static int launch_slim(const void* A, const void* W, void* C, int epi, int M, in
     } while (0)
     if (is_gated(epi)) {
         dim3 grid(N / 32);
-        if (epi == EPI_GATED_BF16) SLIM(2, 16, EPI_GATED_BF16); else SLIM(2, 16, EPI_GATED_GELU_BF16);
+        if (epi == EPI_GATED_BF16) SLIM(2, 16, EPI_GATED_BF16); else if (epi == EPI_GATED_GELU_BF16) SLIM(2, 16, EPI_GATED_GELU_BF16); else SLIM(2, 16, EPI_GATED_CLAMP_BF16);
     } else if (slim_strip_rows(M, N, epi) == 16) {
         dim3 grid((N + 15) / 16);
         if (epi == EPI_STORE_F32) SLIM(1, 16, EPI_STORE_F32); else if (epi == EPI_ADD_F32) SLIM(1, 16, EPI_ADD_F32); else SLIM(1, 16, EPI_STORE_BF16);
@@ -1669,7 +1685,7 @@ static int launch_skinny(const void* A, const void* W, void* C, int epi, int M, 
         GI_REQUIRE(norm_out.scaled == nullptr && rope == nullptr, "gemm_bf16: a product this wide does not hand a norm on, or its rows to the cache");
         const int k_per_split = K;
         dim3 grid((N + 63) / 64, 1);
-        if (epi == EPI_GATED_BF16) SKINNY_MT(EPI_GATED_BF16, false); else if (epi == EPI_GATED_GELU_BF16) SKINNY_MT(EPI_GATED_GELU_BF16, false); else if (epi == EPI_STORE_F32) SKINNY_MT(EPI_STORE_F32, false);
+        if (epi == EPI_GATED_BF16) SKINNY_MT(EPI_GATED_BF16, false); else if (epi == EPI_GATED_GELU_BF16) SKINNY_MT(EPI_GATED_GELU_BF16, false); else if (epi == EPI_GATED_CLAMP_BF16) SKINNY_MT(EPI_GATED_CLAMP_BF16, false); else if (epi == EPI_STORE_F32) SKINNY_MT(EPI_STORE_F32, false);
         else if (epi == EPI_ADD_F32) SKINNY_MT(EPI_ADD_F32, false); else SKINNY_MT(EPI_STORE_BF16, false);
         GI_CHECK_LAUNCH("gemm_bf16 (skinny)");
         return 0;
@@ -1705,6 +1721,7 @@ static int large_norm_parts(int M, int N, int K) {
 // `rope` != null: the sums are those of an attention layer's q/k/v product and go where it says (`epi` is then not looked at).
 static int launch_large(const void* A, const void* W, void* C, int epi, int M, int N, int K, long lda, long ldw, long ldc, float* scratch,
                         long scratch_floats, NormIn norm_in, const RopeStore* rope, hipStream_t stream, NormOut norm_out = NO_NORM_OUT) {
+    const NormIn limit_in = {nullptr, 0, 0.f, 1, norm_in.limit};          // no norm to finish, the clamped gate's limit alone
 #define PIPED(BM_, BN_, WM_, WN_, ST_, EPI_, OUT_, LDC_, SPLITS_, KPS_, SLAB_, NORM_, ROPE_)                                            \
     do {                                                                                                                                \
         constexpr int bytes = ST_ * (BM_ + BN_) * 128;                                                                                  \
@@ -1725,7 +1742,8 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
         else if (epi == EPI_ADD_F32) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_ADD_F32, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);                \
         else if (epi == EPI_STORE_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_STORE_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);          \
         else if (epi == EPI_GATED_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);          \
-        else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_GELU_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE);                                \
+        else if (epi == EPI_GATED_GELU_BF16) PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_GELU_BF16, C, ldc, 1, K, 0L, NO_NORM_IN, NO_ROPE); \
+        else PIPED(BM_, BN_, WM_, WN_, ST_, EPI_GATED_CLAMP_BF16, C, ldc, 1, K, 0L, limit_in, NO_ROPE);                                 \
     } while (0)
     const int splits = gi_gemm_bf16_piped_splits(M, N, K);
     if (splits > 1) {                              // few tiles: k is shared out, the sums are finished by the reduce kernel
@@ -1763,7 +1781,7 @@ static int launch_large(const void* A, const void* W, void* C, int epi, int M, i
     } while (0)
         GI_REQUIRE(lda < (1L << 22) && ldw < (1L << 22), "gemm_bf16: row strides %ld, %ld are too large for the tile-relative addressing", lda, ldw);
         if (epi == EPI_STORE_F32) PINGPONG(EPI_STORE_F32); else if (epi == EPI_ADD_F32) PINGPONG(EPI_ADD_F32);
-        else if (epi == EPI_STORE_BF16) PINGPONG(EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) PINGPONG(EPI_GATED_BF16); else PINGPONG(EPI_GATED_GELU_BF16);
+        else if (epi == EPI_STORE_BF16) PINGPONG(EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) PINGPONG(EPI_GATED_BF16); else if (epi == EPI_GATED_GELU_BF16) PINGPONG(EPI_GATED_GELU_BF16); else PINGPONG(EPI_GATED_CLAMP_BF16);
 #undef PINGPONG
         GI_CHECK_LAUNCH("gemm_bf16 (pingpong)");
         return 0;
@@ -1809,7 +1827,7 @@ GI_API int gi_gemm_bf16_takes_norm(int M, int N, int K, int gated) {
 // row's sum of x^2; the results are multiplied by rsqrt(sum / K + eps).  scaled_out != null (needs accumulate onto 32-bit C):
 // beside C += A W^T, scaled_out [M, ld_scaled] = bfloat16(g * C) and squares_out [M, gi_gemm_bf16_norm_parts(M, N, K)] = the
 // pieces of the rows' sums of C^2, for the next product.  Where the two queries above say no, it fails.
-GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, int M, int N, int K, long lda,
+GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, float gate_limit, int M, int N, int K, long lda,
                                 long ldw, long ldc, float* scratch, long scratch_floats, const float* squares_in, int parts_in, float eps,
                                 const float* g, void* scaled_out, long ld_scaled, float* squares_out, hipStream_t stream) {
     GI_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: M %d, N %d, K %d must be positive", M, N, K);
@@ -1819,7 +1837,7 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
     int epi = epilogue_of(c_dtype, accumulate);
     if (gated) {
         GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16 && !accumulate, "gemm_bf16: the gated product needs N %% 32 == 0 and a bfloat16 output");
-        epi = gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
+        epi = gated == 3 ? EPI_GATED_CLAMP_BF16 : gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
     GI_REQUIRE(squares_in == nullptr || (parts_in > 0 && gi_gemm_bf16_takes_norm(M, N, K, gated)),
@@ -1827,7 +1845,7 @@ GI_API int gi_gemm_bf16_handing(const void* A, const void* W, void* C, int c_dty
     GI_REQUIRE(scaled_out == nullptr || (epi == EPI_ADD_F32 && g != nullptr && squares_out != nullptr && ld_scaled >= N && gi_gemm_bf16_norm_parts(M, N, K) > 0),
                "gemm_bf16: handing a norm on needs a product that adds onto 32-bit rows, of sizes that allow it (M %d, N %d, K %d), the norm's weights and "
                "room for the sums of squares", M, N, K);
-    const NormIn norm_in = {squares_in, parts_in, eps, K};
+    const NormIn norm_in = {squares_in, parts_in, eps, K, gate_limit};
     const NormOut norm_out = {g, (bf16_t*)scaled_out, ld_scaled, squares_out};
     if (takes_slim(M, N, K)) {
         GI_REQUIRE(squares_in == nullptr || parts_in <= slim_max_parts(M), "gemm_bf16: %d pieces of a sum of squares, at most %d", parts_in, slim_max_parts(M));
@@ -1891,7 +1909,7 @@ GI_API int gi_gemm_bf16_qkv_rope_store(const void* A, const void* W, int M, int 
 
 // `gated` != 0: W is [gate; up] interleaved in groups of 16 rows (N rows in all, a multiple of 32)
 // and C is bfloat16 [M, N/2] = silu(gate) * up.
-GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, int M, int N, int K, long lda,
+GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int accumulate, int gated, float gate_limit, int M, int N, int K, long lda,
                         long ldw, long ldc, float* scratch, long scratch_floats, hipStream_t stream) {
     GI_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: M %d, N %d, K %d must be positive", M, N, K);
     GI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_bf16: K %d and the row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
@@ -1900,26 +1918,27 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
     int epi = epilogue_of(c_dtype, accumulate);
     if (gated) {
         GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16 && !accumulate, "gemm_bf16: the gated product needs N %% 32 == 0 and a bfloat16 output");
-        epi = gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
+        epi = gated == 3 ? EPI_GATED_CLAMP_BF16 : gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16: output dtype %d with accumulate %d is not supported", c_dtype, accumulate);
 
-    if (takes_slim(M, N, K)) return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, NO_NORM_IN, NO_NORM_OUT, stream);
+    const NormIn plain_in = {nullptr, 0, 0.f, 1, gate_limit};          // no norm to finish; the clamped gate's limit
+    if (takes_slim(M, N, K)) return launch_slim(A, W, C, epi, M, N, K, lda, ldw, ldc, plain_in, NO_NORM_OUT, stream);
 
-    if (takes_slim_tiles(M, N, K, epi)) return launch_slim_tiles(A, W, C, epi, M, N, K, lda, ldw, ldc, NO_NORM_IN, NO_NORM_OUT, stream);
-    if (M <= SKINNY_MAX_ROWS) return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, NO_NORM_IN, NO_NORM_OUT, stream);
+    if (takes_slim_tiles(M, N, K, epi)) return launch_slim_tiles(A, W, C, epi, M, N, K, lda, ldw, ldc, plain_in, NO_NORM_OUT, stream);
+    if (M <= SKINNY_MAX_ROWS) return launch_skinny(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, plain_in, NO_NORM_OUT, stream);
 
     GI_REQUIRE((M + 63) / 64 <= 65535, "gemm_bf16: M %d is too large", M);
-    if (K % PK == 0 && N >= 128) return launch_large(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, NO_NORM_IN, nullptr, stream);
-#define TILED(BM_, EPI_) gemm_bf16_tiled_kernel<BM_, EPI_><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc)
+    if (K % PK == 0 && N >= 128) return launch_large(A, W, C, epi, M, N, K, lda, ldw, ldc, scratch, scratch_floats, plain_in, nullptr, stream);
+#define TILED(BM_, EPI_) gemm_bf16_tiled_kernel<BM_, EPI_><<<grid, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, gate_limit)
     if ((long)((M + 127) / 128) * ((N + BN - 1) / BN) < 512) {   // few tiles: smaller ones fill more of the chip
         dim3 grid((N + BN - 1) / BN, (M + 63) / 64);
         if (epi == EPI_STORE_F32) TILED(64, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(64, EPI_ADD_F32);
-        else if (epi == EPI_STORE_BF16) TILED(64, EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) TILED(64, EPI_GATED_BF16); else TILED(64, EPI_GATED_GELU_BF16);
+        else if (epi == EPI_STORE_BF16) TILED(64, EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) TILED(64, EPI_GATED_BF16); else if (epi == EPI_GATED_GELU_BF16) TILED(64, EPI_GATED_GELU_BF16); else TILED(64, EPI_GATED_CLAMP_BF16);
     } else {
         dim3 grid((N + BN - 1) / BN, (M + 127) / 128);
         if (epi == EPI_STORE_F32) TILED(128, EPI_STORE_F32); else if (epi == EPI_ADD_F32) TILED(128, EPI_ADD_F32);
-        else if (epi == EPI_STORE_BF16) TILED(128, EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) TILED(128, EPI_GATED_BF16); else TILED(128, EPI_GATED_GELU_BF16);
+        else if (epi == EPI_STORE_BF16) TILED(128, EPI_STORE_BF16); else if (epi == EPI_GATED_BF16) TILED(128, EPI_GATED_BF16); else if (epi == EPI_GATED_GELU_BF16) TILED(128, EPI_GATED_GELU_BF16); else TILED(128, EPI_GATED_CLAMP_BF16);
     }
 #undef TILED
     GI_CHECK_LAUNCH("gemm_bf16 (tiled)");
@@ -1928,7 +1947,7 @@ GI_API int gi_gemm_bf16(const void* A, const void* W, void* C, int c_dtype, int 
 
 // C[rows of tile t] = A[rows of tile t] * W[tile_group[t]]^T for every tile t of 128 rows of A that is in use (see the kernel).  M rows
 // of A and C exist (a multiple of 128); W is [groups][N][K].  Output: float32 stored, bfloat16 stored, or the gated form.
-GI_API int gi_gemm_bf16_grouped(const void* A, const void* W, void* C, int c_dtype, int gated, int M, int N, int K, long lda, long ldw, long ldc,
+GI_API int gi_gemm_bf16_grouped(const void* A, const void* W, void* C, int c_dtype, int gated, float gate_limit, int M, int N, int K, long lda, long ldw, long ldc,
                                 const int* tile_group, long group_stride, hipStream_t stream) {
     GI_REQUIRE(M > 0 && M % 128 == 0 && N >= 128 && K > 0 && K % PK == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K && ldc >= (gated ? N / 2 : N)
                && group_stride % 8 == 0 && M / 128 <= 65535,
@@ -1937,7 +1956,7 @@ GI_API int gi_gemm_bf16_grouped(const void* A, const void* W, void* C, int c_dty
     int epi = epilogue_of(c_dtype, 0);
     if (gated) {
         GI_REQUIRE(N % 32 == 0 && c_dtype == GI_BF16, "gemm_bf16_grouped: the gated product needs N %% 32 == 0 and a bfloat16 output");
-        epi = gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
+        epi = gated == 3 ? EPI_GATED_CLAMP_BF16 : gated == 2 ? EPI_GATED_GELU_BF16 : EPI_GATED_BF16;
     }
     GI_REQUIRE(epi >= 0, "gemm_bf16_grouped: output dtype %d is not supported", c_dtype);
     constexpr int bytes = 2 * 256 * 128;
@@ -1950,12 +1969,13 @@ GI_API int gi_gemm_bf16_grouped(const void* A, const void* W, void* C, int c_dty
                 return gi_fail("gemm_bf16_grouped: cannot reserve %d bytes of LDS", bytes);                                                         \
             raised = true;                                                                                                                          \
         }                                                                                                                                           \
-        gemm_bf16_grouped_kernel<EPI_><<<grid, 256, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, tile_group, group_stride); \
+        gemm_bf16_grouped_kernel<EPI_><<<grid, 256, bytes, stream>>>((const bf16_t*)A, (const bf16_t*)W, C, M, N, K, lda, ldw, ldc, tile_group, group_stride, gate_limit); \
     } while (0)
     if (epi == EPI_STORE_F32) GROUPED(EPI_STORE_F32);
     else if (epi == EPI_STORE_BF16) GROUPED(EPI_STORE_BF16);
     else if (epi == EPI_GATED_BF16) GROUPED(EPI_GATED_BF16);
-    else GROUPED(EPI_GATED_GELU_BF16);
+    else if (epi == EPI_GATED_GELU_BF16) GROUPED(EPI_GATED_GELU_BF16);
+    else GROUPED(EPI_GATED_CLAMP_BF16);
 #undef GROUPED
     GI_CHECK_LAUNCH("gemm_bf16 (grouped)");
     return 0;

@@ -57,7 +57,7 @@ _SIGNATURES = {
     "gi_experts_place": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "gi_experts_gather": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_void_p],
     "gi_experts_combine": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_int, c_void_p],
-    "gi_gemm_bf16_grouped": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
+    "gi_gemm_bf16_grouped": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_experts_down": [c_void_p, c_int, c_long, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gi_xielu": [c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_void_p, c_void_p],
     "gi_delta_prepare": [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p,
@@ -82,16 +82,16 @@ _SIGNATURES = {
     "gi_mlstm_scan": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p, c_int, c_void_p,
                       c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
     "gi_head_norm_gate": [c_void_p, c_long, c_void_p, c_void_p, c_long, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p],
-    "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
+    "gi_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long, c_void_p],
     "gi_attention_prompt_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
-                                 c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_void_p],
+                                 c_float, c_int, c_void_p, c_void_p, c_int, c_void_p, c_long, c_int, c_void_p, c_void_p, c_long, c_float, c_void_p],
     "gi_attention_decode_bf16": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                  c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int,
-                                 c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_long, c_void_p],
+                                 c_float, c_int, c_int, c_int, c_void_p, c_void_p, c_long, c_float, c_void_p],
     "gi_random_normal": [c_void_p, c_int, c_long, ctypes.c_ulonglong, ctypes.c_double, ctypes.c_double, c_void_p],
     "gi_probe_stream": [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p],
     "gi_probe_mfma": [c_int, c_void_p, c_int, c_void_p],
-    "gi_gemm_bf16_handing": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long,
+    "gi_gemm_bf16_handing": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p, c_long,
                              c_void_p, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p, c_void_p],
     "gi_gemm_bf16_qkv_rope_store": [c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p,
                                     c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p],
@@ -596,7 +596,7 @@ def xielu(x, out, params):
 ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "swish_clamped": 2}
 # "swish_clamped" takes a number, `limit`: both halves are clamped first, g <- min(g, limit), u <- clamp(u, -limit, limit), and the
 # result is g * sigmoid(1.702 g) * (u + 1).
-FUSED_GATE_ACTIVATIONS = ("silu", "gelu_tanh")        # those the matrix-core products apply in their own last step
+FUSED_GATE_ACTIVATIONS = ("silu", "gelu_tanh", "swish_clamped")        # those the matrix-core products apply in their own last step
 
 
 def act_mul(gate_up, out, activation="silu", limit=0.0):
@@ -1022,7 +1022,7 @@ def decode_attention_shape(n_decode, n_heads, n_kv, hd, span, target_waves=4096,
 
 
 def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, n_heads, n_kv, hd, window=None, scale=None,
-                   target_waves: int = 4096, products=None, chunk=None, sinks=None, gate=None):
+                   target_waves: int = 4096, products=None, chunk=None, sinks=None, gate=None, cap=None):
     """Attention of a step's rows with the matrix-core kernels (bfloat16 cache and out).
 
     `q` holds the rotated queries in bfloat16 and the cache the rows' keys and values; or, for a step
@@ -1039,7 +1039,9 @@ def attention_bf16(q, cache, out, plan: AttentionPlan, positions, slots, table, 
     if gate is not None and not (gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == n and gate.shape[1] >= n_heads and gate.stride(1) == 1):
         raise KernelError("attention: the heads' gates must be float32 [n, heads] with unit inner stride")
     chunk = int(chunk or 0)
-    extras = (chunk, _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0)
+    if cap is not None and not cap > 0:
+        raise KernelError("attention: the scores' cap must be positive")
+    extras = (chunk, _ptr(sinks), _ptr(gate), gate.stride(0) if gate is not None else 0, float(cap or 0.0))
     seen = lambda context, slack: min([context] + ([window + slack] if window else []) + ([chunk + slack] if chunk else []))
     for t, name in ((q, "q"), (cache, "cache"), (out, "out")):
         if not (t is None or t.dtype == torch.bfloat16):
@@ -1109,11 +1111,11 @@ def attention_general(q, cache, out, ctx, table, n_heads, n_kv, hd, *, page_size
     """Attention of a step's rows for layers with any of: value heads of another size, a scale of their own, a mask cut into
     chunks, sinks, a gate per head, capped scores."""
     vd = int(value_dim or hd)
-    if (cap is None and vd == hd and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
-            and (gate is None or gate.dtype == torch.float32)):
+    if (vd == hd and cache.dim() == 5 and q.dtype == torch.bfloat16 and cache.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+            and (gate is None or gate.dtype == torch.float32) and (cap is None or hd <= 128)):          # (capped scores on the matrix cores: tested up to heads of 128)
         plan = _plan_of(ctx)
         if (not plan.n_tiles or attention_bf16_supports(hd, page_size, True)) and (not plan.n_decode or attention_bf16_supports(hd, page_size, False)):
-            return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, chunk=chunk, sinks=sinks, gate=gate)
+            return attention_bf16(q, cache, out, plan, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, chunk=chunk, sinks=sinks, gate=gate, cap=cap)
     return attention_exact(q, cache, out, ctx.row_pos, ctx.row_slot, table, n_heads, n_kv, hd, window, scale, page_size=page_size,
                            value_dim=value_dim, chunk=chunk, sinks=sinks, gate=gate, cap=cap)
 
@@ -1170,10 +1172,11 @@ def gemm_bf16_takes_norm(m, n, k, gated=False) -> bool:
     return bool(lib().gi_gemm_bf16_takes_norm(m, n, k, 1 if gated else 0))
 
 
-def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=None, norm_out=None):
+def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=None, norm_out=None, gate_limit=0.0):
     """out (=|+=) a @ w.T with bfloat16 operands on the matrix cores, float32 sums.
     gated: w is [gate; up] interleaved in groups of 16 rows and out = act(a @ gate.T) * (a @ up.T), bfloat16 [m, n/2]; act is
-    SiLU (gated = True or "silu") or the tanh form of GELU (gated = "gelu_tanh").
+    SiLU (gated = True or "silu"), the tanh form of GELU (gated = "gelu_tanh") or the clamped form (gated = "swish_clamped", with
+    `gate_limit`; see `ACTIVATIONS`).
 
     An RMS norm between two products of a few rows, without a kernel of its own:
     norm_out = (g, scaled, squares), with accumulate: beside out += a @ w.T, scaled = bfloat16(g * out) and squares
@@ -1208,11 +1211,11 @@ def gemm_bf16(a, w, out, accumulate=False, gated=False, checked=False, norm_in=N
                 raise KernelError("gemm: handing a norm on needs a product of a few rows that adds onto float32 rows, float32 weights of the norm, "
                                   "bfloat16 [m, n] for the scaled rows and float32 [m, gemm_bf16_norm_parts] for the sums of squares")
             _dev(g, scaled, squares_out)
-        _call("gi_gemm_bf16_handing", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, gate_code,
+        _call("gi_gemm_bf16_handing", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, gate_code, float(gate_limit),
               m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _ptr(squares_in), squares_in.shape[1] if squares_in is not None else 0, float(eps),
               _ptr(g), _ptr(scaled), scaled.stride(0) if scaled is not None else 0, _ptr(squares_out), _stream())
         return out
-    _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, gate_code,
+    _call("gi_gemm_bf16", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm: out"), 1 if accumulate else 0, gate_code, float(gate_limit),
           m, n, k, a.stride(0), w.stride(0), out.stride(0), _ptr(scratch), n_scratch, _stream())
     return out
 
@@ -1699,7 +1702,7 @@ def route_rows(h, router, top, ids, weights, score="sigmoid", renormalize=False,
           _ptr(logits), logits.stride(0) if logits is not None else 0, _stream())
 
 
-def gemm_bf16_grouped(a, w, out, tile_group, gated=False):
+def gemm_bf16_grouped(a, w, out, tile_group, gated=False, gate_limit=0.0):
     """out[rows of tile t] = a[rows of tile t] @ w[tile_group[t]].T for every tile t of 128 rows with tile_group[t] >= 0: bfloat16 on
     the matrix cores.  a [m, k] with m a multiple of 128, w [groups, n, k], out float32 or bfloat16 [m, n], or, gated (as
     `gemm_bf16`), bfloat16 [m, n / 2].  Tiles with a negative entry are left as they are."""
@@ -1715,7 +1718,7 @@ def gemm_bf16_grouped(a, w, out, tile_group, gated=False):
     gate_code = 0 if not gated else 1 + (0 if gated is True else ACTIVATIONS[gated])
     if _profile is not None:
         _profile.note = (f"{m}x{n}x{k}{' gated' if gated else ''}", 0)
-    _call("gi_gemm_bf16_grouped", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm_bf16_grouped: out"), gate_code, m, n, k, a.stride(0), w.stride(1),
+    _call("gi_gemm_bf16_grouped", a.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out, "gemm_bf16_grouped: out"), gate_code, float(gate_limit), m, n, k, a.stride(0), w.stride(1),
           out.stride(0), tile_group.data_ptr(), w.stride(0), _stream())
     return out
 
@@ -1755,7 +1758,7 @@ def routed_experts(h, w_gate, w_up, w_down, ids, weights, x, accumulate=True, we
         _call("gi_experts_gather", h.data_ptr(), h.stride(0), place.data_ptr(), weights.data_ptr(), 1 if weigh == "input" else 0, n, top, rows.data_ptr(), rows.stride(0),
               width, _stream())
         mid = torch.empty((n_tiles * tile, ff), dtype=torch.bfloat16, device=dev)
-        gemm_bf16_grouped(rows, w_gate, mid, tile_expert, gated=True if activation == "silu" else activation)
+        gemm_bf16_grouped(rows, w_gate, mid, tile_expert, gated=True if activation == "silu" else activation, gate_limit=limit)
         y = torch.empty((n_tiles * tile, width), dtype=torch.float32, device=dev)
         gemm_bf16_grouped(mid, w_down, y, tile_expert)
         _call("gi_experts_combine", y.data_ptr(), y.stride(0), place.data_ptr(), weights.data_ptr(), 1 if weigh == "output" else 0, n, top, x.data_ptr(), x.stride(0),

@@ -17,17 +17,17 @@ from ..kernels import ops
 from .norm import HandedRows, NormedRows
 
 
-def linear(a, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False, gated: bool = False) -> torch.Tensor:
+def linear(a, weight: torch.Tensor, out: torch.Tensor, accumulate: bool = False, gated: bool = False, gate_limit: float = 0.0) -> torch.Tensor:
     """gated: weight is [gate; up] interleaved by `ops.interleave_gate_up` and out = act(gate) * up (bfloat16 only); True or "silu"
-    for SiLU, "gelu_tanh" for the tanh form of GELU."""
+    for SiLU, "gelu_tanh" for the tanh form of GELU, "swish_clamped" (with `gate_limit`) for the clamped form."""
     if isinstance(a, HandedRows):
         if (weight.dtype == torch.bfloat16 and ops.gemm_bf16_supports(a.scaled, weight, out)
                 and ops.gemm_bf16_takes_norm(a.scaled.shape[0], weight.shape[0], weight.shape[1], gated)):
-            return ops.gemm_bf16(a.scaled, weight, out, accumulate, gated, checked=True, norm_in=(a.squares, a.eps))
+            return ops.gemm_bf16(a.scaled, weight, out, accumulate, gated, checked=True, norm_in=(a.squares, a.eps), gate_limit=gate_limit)
     if isinstance(a, NormedRows):
         a = a.materialize()
     if a.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and ops.gemm_bf16_supports(a, weight, out):
-        return ops.gemm_bf16(a, weight, out, accumulate, gated, checked=True)
+        return ops.gemm_bf16(a, weight, out, accumulate, gated, checked=True, gate_limit=gate_limit)
     if gated:
         raise ops.KernelError("the gated product exists for bfloat16 operands only")
     return ops.gemm_exact(a, weight, out, accumulate)

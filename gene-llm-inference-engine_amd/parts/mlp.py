@@ -44,7 +44,7 @@ class SwiGlu(FeedForward):
         T, inter = ctx.n_rows, self.spec.intermediate_size
         if self.fused:
             mid = torch.empty((T, inter), dtype=torch.bfloat16, device=ctx.device)
-            linear(h, self.w_gate_up, mid, gated=self.activation)
+            linear(h, self.w_gate_up, mid, gated=self.activation, gate_limit=self.limit)
         else:
             gate_up = torch.empty((T, 2 * inter), dtype=torch.float32, device=ctx.device)
             linear(h, self.w_gate_up, gate_up)

@@ -545,3 +545,72 @@ def test_the_new_parts_serve_other_designs():
         x = x + (g * torch.sigmoid(g) * (h @ w["up"].T)) @ w["down"].T
     want = P.rms_norm(x, w["nf"], 1e-5) @ w["embed"].T
     assert relative_error(got[0], want) < 2e-5
+
+
+@pytest.mark.parametrize("case", range(10))
+def test_capped_scores_in_the_matrix_core_kernels(case):
+    """Steps drawn at random through the bfloat16 attention kernels with a cap on the scores (both prompt kernels, the decode kernel,
+    keys shared out over workgroups) against a dense 64-bit computation: single rows, short portions and up to 900 rows on top of up
+    to 2,000 cached positions, scores several times the cap, pages on scrambled numbers between pages of NaN."""
+    import random
+    from geneinfer_amd.kernels import ops
+    from geneinfer_amd.parts import StepContext
+    rng = random.Random(300 + case)
+    torch.manual_seed(case)
+    hd = (64, 128)[case % 2]
+    KV = rng.choice([1, 2, 4])
+    H = KV * rng.choice([1, 2, 4])
+    page = rng.choice([16, 32, 64])
+    cap, scale = rng.choice([1.5, 5.0, 30.0]), rng.choice([0.125, 0.5])
+    segs = []
+    for s in range(rng.randrange(1, 5)):
+        kind = rng.random()
+        start = rng.choice([0, 0, rng.randrange(1, 2000)])
+        segs.append((s, start, 1 if kind < 0.3 else rng.randrange(2, 60) if kind < 0.5 else rng.randrange(65, 900)))
+    R, ctxs = len(segs), [st + n for _, st, n in segs]
+    per = [-(-c // page) for c in ctxs]
+    n_pages = sum(per) + 3
+    cache = torch.full((n_pages, 2, KV, page, hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    perm = iter(torch.randperm(n_pages)[:sum(per)].tolist())
+    table = torch.full((R, max(per)), -1, dtype=torch.int32)
+    K, V = [], []
+    for s, c in enumerate(ctxs):
+        k, v = torch.randn(c, KV, hd, device=DEV).bfloat16(), torch.randn(c, KV, hd, device=DEV).bfloat16()
+        K.append(k)
+        V.append(v)
+        for pi in range(per[s]):
+            pg = next(perm)
+            table[s, pi] = pg
+            lo, hi = pi * page, min(c, (pi + 1) * page)
+            bk, bv = torch.zeros(page, KV, hd, dtype=torch.bfloat16, device=DEV), torch.zeros(page, KV, hd, dtype=torch.bfloat16, device=DEV)
+            bk[:hi - lo], bv[:hi - lo] = k[lo:hi], v[lo:hi]
+            cache[pg, 0] = bk.permute(1, 0, 2)
+            cache[pg, 1].view(KV, hd, page).copy_(bv.permute(1, 2, 0))
+    table = table.to(DEV)
+    rows, seg_start, seg_len, seg_pos0, seg_slot = [], [], [], [], []
+    for s, st, n in segs:
+        seg_start.append(len(rows)); seg_len.append(n); seg_pos0.append(st); seg_slot.append(s)
+        rows += [(s, st + i) for i in range(n)]
+    T = len(rows)
+    q = torch.randn(T, H * hd, device=DEV).bfloat16()
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([s for s, _ in rows], dtype=torch.int32, device=DEV)
+    ctx = StepContext(n_rows=T, dtype=torch.bfloat16, device=torch.device(DEV), tokens=pos, row_pos=pos, row_slot=slots, seg_slot=seg_slot, seg_start=seg_start,
+                      seg_len=seg_len, seg_pos0=seg_pos0)
+    out = torch.full((T, H * hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.attention_general(q, cache, out, ctx, table, H, KV, hd, page_size=page, scale=scale, cap=cap)
+    want = torch.zeros(T, H * hd, dtype=F64)
+    at = 0
+    for s, st, n in segs:
+        qq = q[at:at + n].double().cpu().reshape(n, H, hd)
+        k, v = K[s].double().cpu(), V[s].double().cpu()
+        for a in range(H):
+            sc = cap * torch.tanh((qq[:, a] @ k[:, a // (H // KV)].T) * scale / cap)
+            seen = torch.arange(k.shape[0])[None, :] <= (st + torch.arange(n))[:, None]
+            want[at:at + n, a * hd:(a + 1) * hd] = torch.softmax(sc.masked_fill(~seen, float("-inf")), dim=-1) @ v[:, a // (H // KV)]
+        at += n
+    err = relative_error(out, want)
+    assert bool(torch.isfinite(out.float()).all()) and err < 8e-3, f"case {case}: hd {hd} heads {H}:{KV} page {page} cap {cap} scale {scale} segments {segs}: {err}"
+    exact = torch.empty_like(out)
+    ops.attention_exact(q, cache.view(n_pages, -1), exact, pos, slots, table, H, KV, hd, scale=scale, page_size=page, cap=cap)
+    assert relative_error(exact, want) < 8e-3
