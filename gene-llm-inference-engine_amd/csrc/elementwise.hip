@@ -423,6 +423,30 @@ GI_API int gi_rmsnorm_add(const float* y, const void* w, int w_dtype, float* x, 
 constexpr int NRS_MAX_HD = 512;
 constexpr int NRS_NEIGHBOURS = 1, NRS_UNIT_RMS = 2, NRS_NORM_LAST = 4, NRS_NORM_ALL = 8;
 
+// For a norm over all heads of a projection at once (NRS_NORM_ALL): r[t] = {1 / sqrt(mean(q_t^2) + eps), the same of k_t}, the rows with
+// their biases, one workgroup a row; every head's wave of the kernel below then reads its row's number instead of adding up the
+// whole row once more (which at 32 heads of 128 channels tripled that kernel's time).
+__global__ __launch_bounds__(256) void rows_rsqrt_kernel(const float* __restrict__ q, long ldq, int nq, const float* __restrict__ q_bias, const float* __restrict__ k, long ldk,
+                                                        int nk, const float* __restrict__ k_bias, float eps, float* __restrict__ r) {
+    __shared__ float red[4];
+    const size_t t = blockIdx.x;
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < nq; d += 256) {
+        const float x = q_bias ? q[t * ldq + d] + q_bias[d] : q[t * ldq + d];
+        ss = fmaf(x, x, ss);
+    }
+    ss = block_sum<256>(ss, red);
+    if (threadIdx.x == 0) r[2 * t] = 1.0f / sqrtf(ss / (float)nq + eps);
+    if (k == nullptr) return;
+    ss = 0.f;
+    for (int d = threadIdx.x; d < nk; d += 256) {
+        const float x = k_bias ? k[t * ldk + d] + k_bias[d] : k[t * ldk + d];
+        ss = fmaf(x, x, ss);
+    }
+    ss = block_sum<256>(ss, red);
+    if (threadIdx.x == 0) r[2 * t + 1] = 1.0f / sqrtf(ss / (float)nk + eps);
+}
+
 template <typename TQ, typename TC, typename TW>
 __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ v,
                                                             long ldq, long ldk, long ldv, const TW* __restrict__ q_norm, const TW* __restrict__ k_norm,
@@ -433,7 +457,7 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
                                                             const float* __restrict__ q_bias, const float* __restrict__ k_bias,
                                                             const float* __restrict__ v_bias, const float* __restrict__ v_other, long ld_other,
                                                             const float* __restrict__ v_blend, float* __restrict__ v_keep, long ld_keep, int flags,
-                                                            float v_scale) {
+                                                            float v_scale, const float* __restrict__ rows_r) {
     __shared__ float s[NRS_MAX_HD];
     const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
     const int p = pos[t];
@@ -463,18 +487,9 @@ __global__ __launch_bounds__(64) void norm_rope_store_kernel(const float* __rest
         ss = fmaf(x, x, ss);
     }
     const bool normed = w != nullptr || (flags & NRS_UNIT_RMS), norm_last = normed && (flags & NRS_NORM_LAST);
-    int span = hd;
-    if (normed && (flags & NRS_NORM_ALL)) {          // one norm over all heads of the projection: every head's wave sums the whole row, in the same order
-        span = (is_q ? n_heads : n_kv) * hd;
-        const float* all = src - h * hd;
-        ss = 0.f;
-        for (int d = lane; d < span; d += 64) {
-            const float x = bias ? all[d] + bias[d] : all[d];
-            ss = fmaf(x, x, ss);
-        }
-        w = w != nullptr ? w + h * hd : w;
-    }
-    const float r = normed ? 1.0f / sqrtf(wave_sum(ss) / (float)span + eps) : 1.0f;      // (a rotation keeps the sum of squares: the same number in front of it and behind it)
+    const bool whole = normed && (flags & NRS_NORM_ALL);          // one norm over all heads of the projection: the row's number was made beforehand
+    if (whole && w != nullptr) w += h * hd;
+    const float r = whole ? rows_r[2 * (size_t)t + (is_q ? 0 : 1)] : normed ? 1.0f / sqrtf(wave_sum(ss) / (float)hd + eps) : 1.0f;      // (a rotation keeps the sum of squares: the same number in front of it and behind it)
     if (normed && !norm_last) {
         for (int d = lane; d < hd; d += 64) s[d] = w != nullptr ? load_f32(w, d) * (r * s[d]) : r * s[d];
     }
@@ -510,7 +525,13 @@ GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, lo
                               const int* table, int table_stride, void* q_out, int q_dtype, void* cache, int cache_dtype, long page_stride,
                               int page_size, int n_rows, int n_heads, int n_kv, int hd, int vd, const float* q_bias, const float* k_bias,
                               const float* v_bias, const float* v_other, long ld_other, const float* v_blend, float* v_keep, long ld_keep,
-                              int flags, float v_scale, hipStream_t stream) {
+                              int flags, float v_scale, float* rows_r, hipStream_t stream) {
+    if (flags & NRS_NORM_ALL) {
+        GI_REQUIRE(rows_r != nullptr && !(flags & NRS_UNIT_RMS) && q_norm != nullptr && (k == nullptr || k_norm != nullptr),
+                   "norm_rope_store: a norm over whole projections needs its weights and room for two numbers a row");
+        rows_rsqrt_kernel<<<n_rows, 256, 0, stream>>>(q, ldq, n_heads * hd, q_bias, k, ldk, n_kv * hd, k_bias, eps, rows_r);
+        GI_CHECK_LAUNCH("norm_rope_store (rows)");
+    }
     GI_REQUIRE(!(flags & NRS_UNIT_RMS) || (q_norm == nullptr && k_norm == nullptr), "norm_rope_store: heads divided by their root mean square have no norm weights");
     GI_REQUIRE(!(flags & NRS_NEIGHBOURS) || rot % 2 == 0, "norm_rope_store: neighbouring pairs need an even number of turned channels");
     GI_REQUIRE(n_rows > 0 && n_heads > 0 && n_kv > 0 && hd > 0 && hd <= NRS_MAX_HD && vd > 0, "norm_rope_store: bad sizes (rows %d heads %d kv %d hd %d vd %d)",
@@ -526,7 +547,7 @@ GI_API int gi_norm_rope_store(const float* q, const float* k, const float* v, lo
 #define LAUNCH(TQ, TC, TW)                                                                                                                    \
     norm_rope_store_kernel<TQ, TC, TW><<<grid, 64, 0, stream>>>(q, k, v, ldq, ldk, ldv, (const TW*)q_norm, (const TW*)k_norm, eps, cos_t, sin_t, rot, pos, \
                                                                 slot, table, table_stride, (TQ*)q_out, (TC*)cache, page_stride, page_size, n_heads, n_kv, hd, vd, \
-                                                                q_bias, k_bias, v_bias, v_other, ld_other, v_blend, v_keep, ld_keep, flags, v_scale)
+                                                                q_bias, k_bias, v_bias, v_other, ld_other, v_blend, v_keep, ld_keep, flags, v_scale, rows_r)
     if (q_dtype == GI_F32 && cache_dtype == GI_F32 && norm_dtype == GI_F32) LAUNCH(float, float, float);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
     else if (q_dtype == GI_BF16 && cache_dtype == GI_BF16 && norm_dtype == GI_F32) LAUNCH(bf16_t, bf16_t, float);

@@ -10,7 +10,8 @@
 // every row reads its own experts and the weights' bytes are the cost, and the form of 32-bit models.  Every sum is a lane's own
 // share in a fixed order, then the lanes by a butterfly, then the choices one after the other: nothing depends on the batch.
 //
-//   gi_route_rows        the router's product and its choice in one: logits = W_router a per row, 32-bit sums in a fixed order
+//   gi_route_rows        the router's product and its choice in one: logits = W_router a per row, 32-bit sums in a fixed order; rows of
+//                        the matrix behind the experts' (a gate on a shared expert, say) are multiplied along and their products kept
 //
 // For many (row, choice) items in bfloat16 the items are put in the order of their experts, every expert's run filled up to whole
 // tiles of 128 rows, so that one launch of the matrix-core product for grouped rows (gemm_bf16.hip) serves all experts:
@@ -168,12 +169,12 @@ constexpr int ROUTE_MAX_EXPERTS = 64 * ROUTE_PER_LANE;
 template <typename TA, typename TW>
 __global__ __launch_bounds__(256) void route_rows_kernel(const TA* __restrict__ h, long ldh, const TW* __restrict__ router, long ldr, int width, int n_experts, int top,
                                                         int score_kind, int renormalize, float floor, int n_groups, int keep, int* __restrict__ ids, float* __restrict__ weights,
-                                                        float* __restrict__ logits_out, long ldl) {
+                                                        float* __restrict__ logits_out, long ldl, int n_extra, float* __restrict__ extra_out, long lde) {
     __shared__ float zs[ROUTE_MAX_EXPERTS];
     const size_t t = blockIdx.x;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const TA* a = h + t * ldh;
-    for (int e = wave; e < n_experts; e += 4) {
+    for (int e = wave; e < n_experts + n_extra; e += 4) {          // (rows behind the experts': products of the same rows that are no expert's, kept for the caller)
         const TW* w = router + (size_t)e * ldr;
         // a lane takes eight neighbouring columns at a time, four such pieces asked for at once; the columns left over one by one
         float s = 0.f;
@@ -189,8 +190,11 @@ __global__ __launch_bounds__(256) void route_rows_kernel(const TA* __restrict__ 
         for (int d = whole + lane; d < width; d += 64) s = fmaf(load_f32(w, d), load_f32(a, d), s);
         s = wave_sum(s);
         if (lane == 0) {
-            zs[e] = s;
-            if (logits_out != nullptr) logits_out[t * ldl + e] = s;
+            if (e >= n_experts) extra_out[t * lde + (e - n_experts)] = s;
+            else {
+                zs[e] = s;
+                if (logits_out != nullptr) logits_out[t * ldl + e] = s;
+            }
         }
     }
     __syncthreads();
@@ -328,12 +332,14 @@ GI_API int gi_experts_down(const void* mid, int mid_dtype, long ldm, const void*
 }
 
 GI_API int gi_route_rows(const void* h, int h_dtype, long ldh, const void* router, int r_dtype, long ldr, int n_rows, int width, int n_experts, int top, int score_kind,
-                         int renormalize, float floor, int n_groups, int keep, int* ids, float* weights, float* logits, long ldl, hipStream_t stream) {
+                         int renormalize, float floor, int n_groups, int keep, int* ids, float* weights, float* logits, long ldl, int n_extra, float* extra, long lde,
+                         hipStream_t stream) {
+    GI_REQUIRE(n_extra >= 0 && (n_extra == 0 || (extra != nullptr && lde >= n_extra)), "route_rows: %d rows behind the experts' need room for their products", n_extra);
     GI_REQUIRE(groups_fit(n_experts, top, n_groups, keep), "route_rows: %d experts in %d groups of which %d are kept cannot give %d a row", n_experts, n_groups, keep, top);
     GI_REQUIRE(n_rows > 0 && width > 0 && n_experts > 0 && n_experts <= ROUTE_MAX_EXPERTS && top > 0 && top <= n_experts && top <= 64 && ldh >= width && ldr >= width
                && (score_kind == 0 || score_kind == 1) && (logits == nullptr || ldl >= n_experts),
                "route_rows: bad sizes (rows %d, width %d, experts %d, top %d)", n_rows, width, n_experts, top);
-#define LAUNCH(TA, TW) route_rows_kernel<TA, TW><<<n_rows, 256, 0, stream>>>((const TA*)h, ldh, (const TW*)router, ldr, width, n_experts, top, score_kind, renormalize, floor, n_groups, keep, ids, weights, logits, ldl)
+#define LAUNCH(TA, TW) route_rows_kernel<TA, TW><<<n_rows, 256, 0, stream>>>((const TA*)h, ldh, (const TW*)router, ldr, width, n_experts, top, score_kind, renormalize, floor, n_groups, keep, ids, weights, logits, ldl, n_extra, extra, lde)
     if (h_dtype == GI_BF16 && r_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
     else if (h_dtype == GI_F32 && r_dtype == GI_F32) LAUNCH(float, float);
     else if (h_dtype == GI_F32 && r_dtype == GI_BF16) LAUNCH(float, bf16_t);

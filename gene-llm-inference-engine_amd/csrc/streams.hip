@@ -10,6 +10,7 @@
 //                          the h of the request's row before this one (zeros at position 0), else out = h
 //   gi_streams_write       x_t <- sum_s mix[s, t] x_s + mult * write[t] * y, all copies at once from the old ones
 //                          (mix == nullptr: x_t <- x_t + mult * write[t] * y)
+//   gi_streams_write_norm  the same and, of the new copies, what the layer's next half reads: norm(sum_t read[t] x_t), in one kernel
 //
 // The row before a row is the step's previous row if that belongs to the same request at the position before; otherwise it was
 // the last row of an earlier step, whose h the request's state slot holds (`state` [slots, width], float32).  The workgroup of a
@@ -107,6 +108,168 @@ __global__ __launch_bounds__(256) void streams_norm_shift_kernel(const float* __
     }
 }
 
+// The same in one walk over the row, four neighbouring channels a thread and up to MAXC such pieces a thread kept in registers
+// (widths up to 1024 MAXC, a multiple of 4): the sums u of the row (and of the row before it, where the blend needs that) are made
+// once, squared and added up, and then normed, blended and stored.
+constexpr int MAXC = 8;
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 read_sum4(const float* __restrict__ row, int n, int width, const float* w, int d) {
+    float4 u = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < n; ++s) {
+        const float4 v = ld4(row + (size_t)s * width + d);
+        if (w != nullptr) { u.x = fmaf(w[s], v.x, u.x); u.y = fmaf(w[s], v.y, u.y); u.z = fmaf(w[s], v.z, u.z); u.w = fmaf(w[s], v.w, u.w); }
+        else { u.x += v.x; u.y += v.y; u.z += v.z; u.w += v.w; }
+    }
+    return u;
+}
+__device__ __forceinline__ float squares4(const float4 u, float ss) { return fmaf(u.w, u.w, fmaf(u.z, u.z, fmaf(u.y, u.y, fmaf(u.x, u.x, ss)))); }
+template <typename TW>
+__device__ __forceinline__ float4 weights4(const TW* w, int d) {
+    if (w == nullptr) return float4{1.f, 1.f, 1.f, 1.f};
+    return float4{load_f32(w, d), load_f32(w, d + 1), load_f32(w, d + 2), load_f32(w, d + 3)};
+}
+__device__ __forceinline__ void store4(float* p, const float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16_t* p, const float4 v) { *reinterpret_cast<uint2*>(p) = uint2{f32x2_to_bf16x2(v.x, v.y), f32x2_to_bf16x2(v.z, v.w)}; }
+
+template <typename TW, typename TO>
+__global__ __launch_bounds__(256) void streams_norm_shift_fast_kernel(const float* __restrict__ x, long ldx, int n, int width, const float* __restrict__ read,
+                                                                     const TW* __restrict__ norm_w, float eps, const float* __restrict__ shift,
+                                                                     float* __restrict__ state, long state_stride, const int* __restrict__ pos,
+                                                                     const int* __restrict__ slot, TO* __restrict__ out, long ldo, int n_rows, int mode) {
+    __shared__ float red[4];
+    __shared__ float w_s[MAX_STREAMS];
+    const int t = blockIdx.x;
+    const bool shifts = shift != nullptr;
+    bool last = false, before_in_step = false, before_in_state = false;
+    if (shifts) {
+        const int p = pos[t], sl = slot[t];
+        last = t == n_rows - 1 || slot[t + 1] != sl || pos[t + 1] != p + 1;
+        before_in_step = p > 0 && t > 0 && slot[t - 1] == sl && pos[t - 1] == p - 1;
+        before_in_state = p > 0 && !before_in_step;
+    }
+    const bool writes_out = mode & 1, writes_state = shifts && (mode & 2) && last;
+    if (!writes_out && !writes_state) return;
+    if (read != nullptr && threadIdx.x < n) w_s[threadIdx.x] = read[threadIdx.x];
+    __syncthreads();
+    const float* w = read != nullptr ? w_s : nullptr;
+    const float* row = x + (size_t)t * ldx;
+    const float* row_b = row - ldx;
+    const bool both = writes_out && before_in_step;
+    float4 u[MAXC], ub[MAXC];
+    float ss = 0.f, ss_b = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        const int d = 4 * (threadIdx.x + 256 * i);
+        if (d < width) {
+            u[i] = read_sum4(row, n, width, w, d);
+            ss = squares4(u[i], ss);
+            if (both) {
+                ub[i] = read_sum4(row_b, n, width, w, d);
+                ss_b = squares4(ub[i], ss_b);
+            }
+        }
+    }
+    float r = 1.f, r_b = 1.f;
+    if (norm_w != nullptr) {
+        r = 1.0f / sqrtf(block_sum<256>(ss, red) / (float)width + eps);
+        if (both) r_b = 1.0f / sqrtf(block_sum<256>(ss_b, red) / (float)width + eps);
+    }
+    const int sl = shifts ? slot[t] : 0;
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        const int d = 4 * (threadIdx.x + 256 * i);
+        if (d < width) {
+            const float4 g = weights4(norm_w, d);
+            float4 h = u[i];
+            if (norm_w != nullptr) h = float4{g.x * (r * h.x), g.y * (r * h.y), g.z * (r * h.z), g.w * (r * h.w)};
+            if (writes_out) {
+                float4 o = h;
+                if (shifts) {
+                    float4 hb = {0.f, 0.f, 0.f, 0.f};
+                    if (before_in_step) {
+                        hb = ub[i];
+                        if (norm_w != nullptr) hb = float4{g.x * (r_b * hb.x), g.y * (r_b * hb.y), g.z * (r_b * hb.z), g.w * (r_b * hb.w)};
+                    } else if (before_in_state) {
+                        hb = ld4(state + (size_t)sl * state_stride + d);
+                    }
+                    const float4 sh = ld4(shift + d);
+                    o = float4{fmaf(hb.x - h.x, sh.x, h.x), fmaf(hb.y - h.y, sh.y, h.y), fmaf(hb.z - h.z, sh.z, h.z), fmaf(hb.w - h.w, sh.w, h.w)};
+                }
+                store4(out + (size_t)t * ldo + d, o);
+            }
+            if (writes_state) store4(state + (size_t)sl * state_stride + d, h);
+        }
+    }
+}
+
+// A half's result written into the copies and, on the way, what the layer's next half reads of them: the copies of a row become
+// x_t <- sum_s mix[s, t] x_s + mult * write[t] * y, and out = norm_w * u / sqrt(mean(u^2) + eps) with u = sum_t read[t] x_t of the new
+// copies.  Up to 8 copies, widths as above.
+constexpr int FUSED_MAX_STREAMS = 8;
+template <typename TW, typename TO>
+__global__ __launch_bounds__(256) void streams_write_norm_kernel(float* __restrict__ x, long ldx, int n, int width, const float* __restrict__ y, long ldy,
+                                                                const float* __restrict__ mix, const float* __restrict__ write, float mult,
+                                                                const float* __restrict__ read, const TW* __restrict__ norm_w, float eps, TO* __restrict__ out, long ldo) {
+    __shared__ float red[4];
+    __shared__ float m_s[FUSED_MAX_STREAMS * FUSED_MAX_STREAMS];
+    __shared__ float o_s[FUSED_MAX_STREAMS], r_s[FUSED_MAX_STREAMS];
+    if (mix != nullptr)
+        for (int i = threadIdx.x; i < n * n; i += 256) m_s[i] = mix[i];
+    if (threadIdx.x < n) {
+        o_s[threadIdx.x] = write != nullptr ? mult * write[threadIdx.x] : mult;
+        r_s[threadIdx.x] = read != nullptr ? read[threadIdx.x] : 1.f;
+    }
+    __syncthreads();
+    float* row = x + (size_t)blockIdx.x * ldx;
+    const float* yr = y + (size_t)blockIdx.x * ldy;
+    float4 u[MAXC];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        const int d = 4 * (threadIdx.x + 256 * i);
+        if (d < width) {
+            float4 old[FUSED_MAX_STREAMS];
+#pragma unroll
+            for (int s = 0; s < FUSED_MAX_STREAMS; ++s)
+                if (s < n) old[s] = ld4(row + (size_t)s * width + d);
+            const float4 v = ld4(yr + d);
+            float4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int to = 0; to < FUSED_MAX_STREAMS; ++to) {
+                if (to < n) {
+                    float4 a;
+                    if (mix != nullptr) {
+                        a = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int s = 0; s < FUSED_MAX_STREAMS; ++s)
+                            if (s < n) {
+                                const float m = m_s[s * n + to];
+                                a.x = fmaf(m, old[s].x, a.x); a.y = fmaf(m, old[s].y, a.y); a.z = fmaf(m, old[s].z, a.z); a.w = fmaf(m, old[s].w, a.w);
+                            }
+                    } else {
+                        a = old[to];
+                    }
+                    const float o = o_s[to], rd = r_s[to];
+                    a = float4{fmaf(o, v.x, a.x), fmaf(o, v.y, a.y), fmaf(o, v.z, a.z), fmaf(o, v.w, a.w)};
+                    store4(row + (size_t)to * width + d, a);
+                    acc = float4{fmaf(rd, a.x, acc.x), fmaf(rd, a.y, acc.y), fmaf(rd, a.z, acc.z), fmaf(rd, a.w, acc.w)};
+                }
+            }
+            u[i] = acc;
+            ss = squares4(acc, ss);
+        }
+    }
+    const float r = 1.0f / sqrtf(block_sum<256>(ss, red) / (float)width + eps);
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        const int d = 4 * (threadIdx.x + 256 * i);
+        if (d < width) {
+            const float4 g = weights4(norm_w, d);
+            store4(out + (size_t)blockIdx.x * ldo + d, float4{g.x * (r * u[i].x), g.y * (r * u[i].y), g.z * (r * u[i].z), g.w * (r * u[i].w)});
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void streams_write_kernel(float* __restrict__ x, long ldx, int n, int width, const float* __restrict__ y, long ldy,
                                                            const float* __restrict__ mix, const float* __restrict__ write, float mult) {
     __shared__ float m_s[MAX_STREAMS * MAX_STREAMS];
@@ -179,9 +342,19 @@ GI_API int gi_streams_norm_shift(const float* x, long ldx, int n, int width, con
     GI_REQUIRE(mode >= 1 && mode <= 3 && ((mode & 1) == 0 || out != nullptr), "streams_norm_shift: mode %d", mode);
     GI_REQUIRE(shift != nullptr ? (state != nullptr && pos != nullptr && slot != nullptr && state_stride >= width) : mode == 1,
                "streams_norm_shift: a blend with the row before needs the state slots, positions and slots; without one there is no state to write");
+    // one walk with the row in registers where the sizes and addresses allow it, else the kernel that makes every sum twice; which
+    // of the two serves is a matter of the sizes alone, so a row's numbers never depend on what else the step holds
+    const bool fast = width % 4 == 0 && width <= 1024 * MAXC && ldx % 4 == 0 && ldo % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
+                      (shift == nullptr || (((uintptr_t)shift & 15) == 0 && ((uintptr_t)state & 15) == 0 && state_stride % 4 == 0));
 #define LAUNCH(TW, TO)                                                                                                                                    \
-    streams_norm_shift_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, read, (const TW*)norm_w, eps, shift, state, state_stride, pos, slot, \
-                                                                  (TO*)out, ldo, n_rows, mode)
+    do {                                                                                                                                                  \
+        if (fast)                                                                                                                                         \
+            streams_norm_shift_fast_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, read, (const TW*)norm_w, eps, shift, state, state_stride, pos, \
+                                                                               slot, (TO*)out, ldo, n_rows, mode);                                     \
+        else                                                                                                                                              \
+            streams_norm_shift_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, read, (const TW*)norm_w, eps, shift, state, state_stride, pos, slot, \
+                                                                          (TO*)out, ldo, n_rows, mode);                                                \
+    } while (0)
     if (w_dtype == GI_F32 && out_dtype == GI_F32) LAUNCH(float, float);
     else if (w_dtype == GI_F32 && out_dtype == GI_BF16) LAUNCH(float, bf16_t);
     else if (w_dtype == GI_BF16 && out_dtype == GI_F32) LAUNCH(bf16_t, float);
@@ -200,6 +373,25 @@ GI_API int gi_streams_write(float* x, long ldx, int n, int width, const float* y
     GI_REQUIRE(grid.y <= 65535, "streams_write: rows too long");
     streams_write_kernel<<<grid, 256, 0, stream>>>(x, ldx, n, width, y, ldy, mix, write, mult);
     GI_CHECK_LAUNCH("streams_write");
+    return 0;
+}
+
+GI_API int gi_streams_write_norm_takes(int n, int width) { return n >= 1 && n <= FUSED_MAX_STREAMS && width % 4 == 0 && width <= 1024 * MAXC ? 1 : 0; }
+
+GI_API int gi_streams_write_norm(float* x, long ldx, int n, int width, const float* y, long ldy, const float* mix, const float* write, float mult, const float* read,
+                                 const void* norm_w, int w_dtype, float eps, void* out, int out_dtype, long ldo, int n_rows, hipStream_t stream) {
+    GI_REQUIRE(n_rows > 0 && gi_streams_write_norm_takes(n, width) && ldx >= (long)n * width && ldy >= width && ldo >= width && norm_w != nullptr && out != nullptr,
+               "streams_write_norm: bad sizes (rows %d, %d copies of %d)", n_rows, n, width);
+    GI_REQUIRE(ldx % 4 == 0 && ldy % 4 == 0 && ldo % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0 && ((uintptr_t)out & 15) == 0,
+               "streams_write_norm: rows must start at multiples of 16 bytes");
+#define LAUNCH(TW, TO) streams_write_norm_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, y, ldy, mix, write, mult, read, (const TW*)norm_w, eps, (TO*)out, ldo)
+    if (w_dtype == GI_F32 && out_dtype == GI_F32) LAUNCH(float, float);
+    else if (w_dtype == GI_F32 && out_dtype == GI_BF16) LAUNCH(float, bf16_t);
+    else if (w_dtype == GI_BF16 && out_dtype == GI_F32) LAUNCH(bf16_t, float);
+    else if (w_dtype == GI_BF16 && out_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
+    else return gi_fail("streams_write_norm: unknown dtypes %d, %d", w_dtype, out_dtype);
+#undef LAUNCH
+    GI_CHECK_LAUNCH("streams_write_norm");
     return 0;
 }
 

@@ -40,7 +40,7 @@ _SIGNATURES = {
     "gi_rmsnorm_add_norm": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_long, c_long, c_long, c_void_p],
     "gi_norm_rope_store": [c_void_p, c_void_p, c_void_p, c_long, c_long, c_long, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int,
                            c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int,
-                           c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_float, c_void_p],
+                           c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_float, c_void_p, c_void_p],
     "gi_concat_rows": [c_void_p, c_long, c_int, c_void_p, c_long, c_int, c_void_p, c_int, c_long, c_int, c_void_p],
     "gi_add_weighted": [c_void_p, c_long, c_void_p, c_long, c_float, c_void_p, c_long, c_float, c_int, c_int, c_void_p],
     "gi_add_vector": [c_void_p, c_long, c_void_p, c_int, c_int, c_int, c_void_p],
@@ -53,7 +53,8 @@ _SIGNATURES = {
                     c_void_p, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_float, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
     "gi_route_top": [c_void_p, c_long, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p],
     "gi_experts_gate_up": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
-    "gi_route_rows": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_void_p],
+    "gi_route_rows": [c_void_p, c_int, c_long, c_void_p, c_int, c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p, c_long, c_int, c_void_p, c_long,
+                      c_void_p],
     "gi_experts_place": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p],
     "gi_experts_gather": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_void_p],
     "gi_experts_combine": [c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_long, c_int, c_int, c_void_p],
@@ -76,6 +77,8 @@ _SIGNATURES = {
     "gi_streams_norm_shift": [c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_long,
                               c_int, c_int, c_void_p],
     "gi_streams_write": [c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_float, c_int, c_void_p],
+    "gi_streams_write_norm": [c_void_p, c_long, c_int, c_int, c_void_p, c_long, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_float, c_void_p, c_int, c_long, c_int,
+                              c_void_p],
     "gi_head_gate": [c_void_p, c_int, c_long, c_void_p, c_long, c_int, c_int, c_int, c_void_p],
     "gi_add_rows_gated": [c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_int, c_int, c_void_p],
     "gi_segments": [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p],
@@ -143,6 +146,8 @@ def lib():
         l.gi_latent_attention_tiles_supports.restype = c_int
         l.gi_latent_attention_tiles_prepare.argtypes = []
         l.gi_latent_attention_tiles_prepare.restype = c_int
+        l.gi_streams_write_norm_takes.argtypes = [c_int, c_int]
+        l.gi_streams_write_norm_takes.restype = c_int
         l.gi_streams_max.argtypes = []
         l.gi_streams_max.restype = c_int
         l.gi_probe_mfma_flops.argtypes = [c_int, c_int]
@@ -572,12 +577,14 @@ def norm_rope_store(q, k, v, q_norm, k_norm, eps, cos, sin, rotary_dim, position
     _i32(positions, "norm_rope_store: positions", n)
     _i32(slots, "norm_rope_store: slots", n)
     cache_code = _code(cache, "norm_rope_store: cache") if k is not None else _code(q_out, "norm_rope_store: q_out")
+    rows_r = torch.empty((n, 2), dtype=torch.float32, device=q.device) if norm_all else None          # the rows' 1 / sqrt(mean square + eps), made by a kernel of its own first
     _call("gi_norm_rope_store", q.data_ptr(), _ptr(k), _ptr(v), q.stride(0), k.stride(0) if k is not None else 0, v.stride(0) if v is not None else 0,
           _ptr(q_norm), _ptr(k_norm), norm_code if norm_code is not None else F32, float(eps), _ptr(cos), _ptr(sin), 2 * half, positions.data_ptr(),
           slots.data_ptr(), _ptr(table) if k is not None else None, table.stride(0) if k is not None else 0, q_out.data_ptr(),
           _code(q_out, "norm_rope_store: q_out"), _ptr(cache) if k is not None else None, cache_code, cache.stride(0) if k is not None else 0,
           int(page_size), n, n_heads, n_kv, hd, vd, _ptr(q_bias), _ptr(k_bias), _ptr(v_bias), _ptr(other), other.stride(0) if other is not None else 0,
-          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, (1 if neighbours else 0) | (2 if unit_rms else 0) | (4 if norm_last else 0) | (8 if norm_all else 0), float(v_scale), _stream())
+          _ptr(weight), _ptr(keep), keep.stride(0) if keep is not None else 0, (1 if neighbours else 0) | (2 if unit_rms else 0) | (4 if norm_last else 0) | (8 if norm_all else 0), float(v_scale),
+          _ptr(rows_r), _stream())
 
 
 def xielu(x, out, params):
@@ -1682,24 +1689,29 @@ def experts_down(mid, w_down, ids, weights, x, accumulate=True, weigh_output=Fal
     return x
 
 
-def route_rows(h, router, top, ids, weights, score="sigmoid", renormalize=False, logits=None, groups=None, floor=0.0):
+def route_rows(h, router, top, ids, weights, score="sigmoid", renormalize=False, logits=None, groups=None, floor=0.0, extra=None):
     """The router's product and its choice in one launch: logits = h @ router.T with 32-bit sums in an order that the width alone
-    fixes, then as `route_top` (with its `groups` and `floor`).  logits: float32 [n, experts] to keep them in, or None."""
-    _dev(h, router, ids, weights, logits)
+    fixes, then as `route_top` (with its `groups` and `floor`).  logits: float32 [n, experts] to keep them in, or None.  extra:
+    float32 [n, k]: the router's matrix has k more rows behind the experts', whose products with the rows go there (no expert's
+    logits: they take no part in the choice)."""
+    _dev(h, router, ids, weights, logits, extra)
     n, width = h.shape
-    n_experts = router.shape[0]
+    n_extra = 0 if extra is None else extra.shape[1]
+    if extra is not None:
+        _f32_rows(extra, "route_rows: the products behind the experts'", n)
+    n_experts = router.shape[0] - n_extra
     if score not in ROUTER_SCORES:
         raise KernelError(f"route_rows: unknown score {score!r}; known: {', '.join(ROUTER_SCORES)}")
     if not (1 <= top <= min(n_experts, ROUTER_MAX_TOP) and n_experts <= ROUTER_MAX_EXPERTS):
         raise KernelError(f"route_rows: top {top} of {n_experts} experts is outside what the kernel takes")
-    if not (h.stride(1) == 1 and router.shape == (n_experts, width) and router.stride(1) == 1 and ids.dtype == torch.int32 and ids.shape == (n, top) and ids.is_contiguous()
+    if not (h.stride(1) == 1 and router.shape == (n_experts + n_extra, width) and router.stride(1) == 1 and ids.dtype == torch.int32 and ids.shape == (n, top) and ids.is_contiguous()
             and weights.dtype == torch.float32 and weights.shape == (n, top) and weights.is_contiguous()):
         raise KernelError("route_rows: h [n, width], the router [experts, width], ids int32 and weights float32 [n, top] are needed")
     if logits is not None:
         _f32_rows(logits, "route_rows: logits", n, n_experts)
     _call("gi_route_rows", h.data_ptr(), _code(h, "route_rows: h"), h.stride(0), router.data_ptr(), _code(router, "route_rows: the router"), router.stride(0), n, width,
           n_experts, top, ROUTER_SCORES[score], 1 if renormalize else 0, float(floor), *_router_groups("route_rows", n_experts, top, groups), ids.data_ptr(), weights.data_ptr(),
-          _ptr(logits), logits.stride(0) if logits is not None else 0, _stream())
+          _ptr(logits), logits.stride(0) if logits is not None else 0, n_extra, _ptr(extra), extra.stride(0) if extra is not None else 0, _stream())
 
 
 def gemm_bf16_grouped(a, w, out, tile_group, gated=False, gate_limit=0.0):
@@ -1834,6 +1846,35 @@ def streams_write(x, n_streams, y, mix, write, mult=1.0):
         raise KernelError("streams_write: the writing weights must be float32 [n]")
     _call("gi_streams_write", x.data_ptr(), x.stride(0), n_streams, width, y.data_ptr(), y.stride(0), _ptr(mix), _ptr(write), float(mult), rows, _stream())
     return x
+
+
+def streams_write_norm_takes(n_streams, width) -> bool:
+    """Whether `streams_write_norm` takes these sizes (a few copies, a width the kernel keeps in registers)."""
+    return bool(lib().gi_streams_write_norm_takes(int(n_streams), int(width)))
+
+
+def streams_write_norm(x, n_streams, y, mix, write, mult, read, norm_weight, eps, out):
+    """`streams_write` and, of the new copies, out = norm_weight * u / sqrt(mean(u^2) + eps) with u = sum_t read[t] x_t (read None: the
+    plain sum): a half's result into the copies and the next half's input out of them, in one kernel."""
+    _dev(x, y, mix, write, read, norm_weight, out)
+    rows = x.shape[0]
+    width = x.shape[1] // n_streams
+    _f32_rows(x, "streams_write_norm: x", rows, n_streams * width)
+    _f32_rows(y, "streams_write_norm: y", rows, width)
+    if not streams_write_norm_takes(n_streams, width):
+        raise KernelError(f"streams_write_norm: {n_streams} copies of {width} channels are not taken")
+    if mix is not None and not (mix.dtype == torch.float32 and mix.is_contiguous() and mix.shape == (n_streams, n_streams)):
+        raise KernelError("streams_write_norm: the mixing matrix must be float32 [n, n]")
+    for v, what in ((write, "writing"), (read, "reading")):
+        if v is not None and not (v.dtype == torch.float32 and v.is_contiguous() and v.numel() == n_streams):
+            raise KernelError(f"streams_write_norm: the {what} weights must be float32 [n]")
+    if not (norm_weight.shape == (width,) and norm_weight.is_contiguous() and out.shape == (rows, width) and out.stride(1) == 1):
+        raise KernelError("streams_write_norm: the norm's weights must be [width] and out [rows, width]")
+    if x.stride(0) % 4 or y.stride(0) % 4 or out.stride(0) % 4 or x.data_ptr() % 16 or y.data_ptr() % 16 or out.data_ptr() % 16:
+        raise KernelError("streams_write_norm: rows must start at multiples of 16 bytes")
+    _call("gi_streams_write_norm", x.data_ptr(), x.stride(0), n_streams, width, y.data_ptr(), y.stride(0), _ptr(mix), _ptr(write), float(mult), _ptr(read),
+          norm_weight.data_ptr(), _code(norm_weight, "streams_write_norm: norm"), float(eps), out.data_ptr(), _code(out, "streams_write_norm: out"), out.stride(0), rows, _stream())
+    return out
 
 
 def head_gate(a, gate, n_heads, vd):

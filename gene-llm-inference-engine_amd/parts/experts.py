@@ -78,14 +78,13 @@ class RoutedExperts(FeedForward):
         rows = h.materialize() if isinstance(h, NormedRows) else h
         ids = torch.empty((T, s.top), dtype=torch.int32, device=dev)
         weights = torch.empty((T, s.top), dtype=torch.float32, device=dev)
-        ops.route_rows(rows, self.router, s.top, ids, weights, s.score, s.renormalize, groups=self.groups, floor=self.floor)
+        gate = torch.empty((T, 1), dtype=torch.float32, device=dev) if self.shared_gated else None          # (its logit comes out of the router's product)
+        ops.route_rows(rows, self.router_all, s.top, ids, weights, s.score, s.renormalize, groups=self.groups, floor=self.floor, extra=gate)
         ops.routed_experts(rows, self.w_gate, self.w_up, self.w_down, ids, weights, residual, accumulate=not overwrite, weigh=s.weigh, activation=s.activation,
                            limit=self.limit)
         if self.shared is not None and not self.shared_gated:
             self.shared.forward(rows, residual, ctx)
         elif self.shared is not None:          # its result in rows of its own, added times the row's gate
-            gate = torch.empty((T, 1), dtype=torch.float32, device=dev)
-            ops.gemm_exact(rows, self.router_all[s.n_experts:], gate)
             if getattr(self.shared, "can_overwrite", False):
                 y = torch.empty_like(residual)
                 self.shared.forward(rows, y, ctx, overwrite=True)

@@ -112,7 +112,8 @@ class _Access:
 
 class MultiStreamBlock:
     stream_aware = True               # its x is [T, n_streams * hidden]
-    FUSE = True                       # the copies' sum, the norm and the blend with the row before in one kernel (off: one after the other)
+    FUSE = True                       # the copies' sum, the norm and the blend with the row before in one kernel, and the mixer's result written into
+                                      # the copies together with the feed-forward's input read out of them (off: one after the other)
 
     def __init__(self, spec, tensors, dtype, device):
         self.spec = spec
@@ -196,10 +197,19 @@ class MultiStreamBlock:
         else:
             h = self._input(x, ctx, self.mixer_norm, self.mixer, self.mixer_access)
             y = self._run(self.mixer, h, ctx, cache)
-        self._output(x, y, self.mixer_access)
+        h = None
+        if (self.feed_forward is not None and self.FUSE and type(self.feed_forward_norm) is RmsNorm and ctx.trace is None
+                and ops.streams_write_norm_takes(self.n_streams, x.shape[1] // self.n_streams)):
+            # the mixer's result into the copies and the feed-forward's input out of them in one kernel
+            a, b = self.mixer_access, self.feed_forward_access
+            h = torch.empty((ctx.n_rows, x.shape[1] // self.n_streams), dtype=getattr(self.feed_forward, "in_dtype", ctx.dtype), device=x.device)
+            ops.streams_write_norm(x, self.n_streams, y, a.mix, a.write, self.scale, b.read, self.feed_forward_norm.weight, self.feed_forward_norm.eps, h)
+        else:
+            self._output(x, y, self.mixer_access)
         self._traced("attn_out", x, ctx)
         if self.feed_forward is not None:
-            h = self._input(x, ctx, self.feed_forward_norm, self.feed_forward, self.feed_forward_access)
+            if h is None:
+                h = self._input(x, ctx, self.feed_forward_norm, self.feed_forward, self.feed_forward_access)
             y = self._run(self.feed_forward, h, ctx)
             self._output(x, y, self.feed_forward_access)
         self._traced("ffn_out", x, ctx)

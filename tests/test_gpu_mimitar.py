@@ -141,6 +141,40 @@ def test_the_copies_written_back_and_the_start(n, width):
     assert torch.equal(ops.streams_spread(x0, torch.empty(6, n * width, device=DEV), n), x0.repeat(1, n))
 
 
+@pytest.mark.parametrize("n, width, out_dtype", [(1, 64, torch.float32), (3, 192, torch.float32), (4, 2048, torch.bfloat16), (8, 36, torch.float32)])
+def test_a_result_written_into_the_copies_and_the_next_input_read_out_of_them_in_one_kernel(n, width, out_dtype):
+    from geneinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(n * width + 1)
+    x, y = torch.randn(7, n * width, generator=g), torch.randn(7, width, generator=g)
+    mix, write, read = torch.eye(n) + 0.3 * torch.randn(n, n, generator=g), torch.randn(n, generator=g), torch.randn(n, generator=g)
+    norm_w = 1 + 0.1 * torch.randn(width, generator=g)
+    assert ops.streams_write_norm_takes(n, width) and not ops.streams_write_norm_takes(9, width) and not ops.streams_write_norm_takes(n, width + 1)
+    new = P.write_streams(x.double().reshape(7, n, width).transpose(0, 1), y.double(), mix.double(), write.double(), 0.7)
+    want = P.rms_norm(P.read_streams(new, read.double()), norm_w.double(), 1e-5)
+    xd, out = x.to(DEV), torch.empty(7, width, dtype=out_dtype, device=DEV)
+    ops.streams_write_norm(xd, n, y.to(DEV), mix.to(DEV), write.to(DEV), 0.7, read.to(DEV), norm_w.to(DEV), 1e-5, out)
+    assert relative_error(xd, new.transpose(0, 1).reshape(7, n * width)) < 1e-6
+    assert relative_error(out, want) < (1e-5 if out_dtype == torch.float32 else 6e-3)
+    # the two kernels it stands for give the same copies, bit for bit, and the same rows up to the order of the sums
+    x2 = ops.streams_write(x.to(DEV), n, y.to(DEV), mix.to(DEV), write.to(DEV), 0.7)
+    assert torch.equal(x2, xd)
+    out2 = ops.streams_norm_shift(x2, n, torch.empty_like(out), read=read.to(DEV), norm_weight=norm_w.to(DEV), eps=1e-5)
+    assert relative_error(out2, out) < (1e-6 if out_dtype == torch.float32 else 1e-2)
+
+
+def test_products_behind_the_experts_come_out_of_the_router_s_kernel():
+    from geneinfer_amd.kernels import ops
+    g = torch.Generator().manual_seed(11)
+    for dtype in (torch.float32, torch.bfloat16):
+        h, router = torch.randn(20, 72, generator=g).to(dtype), torch.randn(6 + 2, 72, generator=g).to(dtype)
+        ids, weights = torch.empty(20, 2, dtype=torch.int32, device=DEV), torch.empty(20, 2, device=DEV)
+        ids2, weights2, extra = torch.empty_like(ids), torch.empty_like(weights), torch.empty(20, 2, device=DEV)
+        ops.route_rows(h.to(DEV), router.to(DEV)[:6], 2, ids, weights, "softmax", True, groups=(3, 2))
+        ops.route_rows(h.to(DEV), router.to(DEV), 2, ids2, weights2, "softmax", True, groups=(3, 2), extra=extra)
+        assert torch.equal(ids, ids2) and torch.equal(weights, weights2)
+        assert relative_error(extra, h.double() @ router.double()[6:].T) < 1e-6
+
+
 @pytest.mark.parametrize("experts, top, groups, keep", [(6, 2, 3, 2), (16, 4, 4, 3), (8, 2, 2, 1), (4, 1, 4, 2), (64, 8, 8, 4), (130, 4, 10, 3), (12, 12, 3, 3), (9, 2, 1, 1)])
 def test_the_router_chooses_among_the_best_groups(experts, top, groups, keep):
     from geneinfer_amd.kernels import ops
