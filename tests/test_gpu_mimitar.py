@@ -541,6 +541,18 @@ def test_replay_through_the_command_line(folders, tmp_path, dtype):
             assert_within_bfloat16_noise(mine, lambda p: exact[p], lambda p: rounded[p], f"replay {rid}")
 
 
+def test_generation_from_the_command_line_on_random_weights():
+    """bin/gi_generate on the shipped example configuration, random weights, greedy: runs, and twice the same."""
+    import subprocess
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    cmd = [str(root / "bin" / "gi_generate"), "--config", str(root / "configs" / "mimitar-small.json"), "--random-seed", "3", "--prompt-ids", "5 17 3 999 4",
+           "--steps", "24", "--temperature", "0"]
+    runs = [subprocess.run(cmd, capture_output=True, text=True, timeout=280) for _ in range(2)]
+    assert all(r.returncode == 0 for r in runs), runs[0].stderr[-2000:]
+    assert runs[0].stdout == runs[1].stdout and len(runs[0].stdout.split()) >= 20
+
+
 def test_the_new_parts_serve_other_designs():
     """The token-shift mixer under the ordinary pre-norm block around a Llama attention, and a norm with weights stored around zero:
     built from specs alone, without a Mimitar configuration, and run under two cuts with equal bits."""
