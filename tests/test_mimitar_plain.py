@@ -1,5 +1,5 @@
 """What fixes the plain Mimitar implementation (`plain_mimitar.py`) and the configuration class, on the CPU: each mechanism against a
-second formulation or a case worked by hand, the configuration's reading, refusals and round trip, and the list of tensors a
+second formulation or a case worked by hand, the configuration's reading, its refusals and what it writes back, and the list of tensors a
 configuration asks for against the folders the tests write."""
 import itertools
 import math
