@@ -196,8 +196,9 @@ class MimitarConfig:
                 j = layer.weights_of
                 if not 0 <= j < len(layers) or j == i or layers[j].weights_of is not None:
                     raise ConfigError(f"config.json: layer {i} uses the weights of layer {j}, which must be another layer with weights of its own")
-                if (layers[j].mixer, layers[j].mlp) != (layer.mixer, layer.mlp):
-                    raise ConfigError(f"config.json: layer {i} uses the weights of layer {j} but is not described as that layer is")
+                if (type(layers[j].mixer), type(layers[j].mlp)) != (type(layer.mixer), type(layer.mlp)):
+                    raise ConfigError(f"config.json: layer {i} uses the weights of layer {j} but is another kind of layer")
+                layers[i] = MimitarLayer(layers[j].mixer, layers[j].mlp, j)          # (it runs as the layer whose weights it uses)
         optional = lambda key, default, **kw: default if cfg.get(key) is None else _number(cfg, key, "the model", **kw)
         return cls(vocab=_int(cfg, "vocab", "the model"), width=_int(cfg, "width", "the model"), norm_eps=_number(cfg.get("norm"), "eps", "'norm'"),
                    layers=tuple(layers), streams=1 if cfg.get("streams") is None else _int(cfg, "streams", "the model"),
