@@ -113,12 +113,26 @@ __global__ __launch_bounds__(256) void streams_norm_shift_kernel(const float* __
 // once, squared and added up, and then normed, blended and stored.
 constexpr int MAXC = 8;
 __device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+// NS > 0: the number of copies is known where the kernel is compiled (1, 2 or 4: all of a row's loads go out at once, no loop over
+// them); NS = 0: any number.  The sums are the same numbers in the same order either way.
+template <int NS>
 __device__ __forceinline__ float4 read_sum4(const float* __restrict__ row, int n, int width, const float* w, int d) {
     float4 u = {0.f, 0.f, 0.f, 0.f};
-    for (int s = 0; s < n; ++s) {
-        const float4 v = ld4(row + (size_t)s * width + d);
-        if (w != nullptr) { u.x = fmaf(w[s], v.x, u.x); u.y = fmaf(w[s], v.y, u.y); u.z = fmaf(w[s], v.z, u.z); u.w = fmaf(w[s], v.w, u.w); }
-        else { u.x += v.x; u.y += v.y; u.z += v.z; u.w += v.w; }
+    if constexpr (NS > 0) {
+        float4 v[NS];
+#pragma unroll
+        for (int s = 0; s < NS; ++s) v[s] = ld4(row + (size_t)s * width + d);
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            if (w != nullptr) { u.x = fmaf(w[s], v[s].x, u.x); u.y = fmaf(w[s], v[s].y, u.y); u.z = fmaf(w[s], v[s].z, u.z); u.w = fmaf(w[s], v[s].w, u.w); }
+            else { u.x += v[s].x; u.y += v[s].y; u.z += v[s].z; u.w += v[s].w; }
+        }
+    } else {
+        for (int s = 0; s < n; ++s) {
+            const float4 v = ld4(row + (size_t)s * width + d);
+            if (w != nullptr) { u.x = fmaf(w[s], v.x, u.x); u.y = fmaf(w[s], v.y, u.y); u.z = fmaf(w[s], v.z, u.z); u.w = fmaf(w[s], v.w, u.w); }
+            else { u.x += v.x; u.y += v.y; u.z += v.z; u.w += v.w; }
+        }
     }
     return u;
 }
@@ -131,7 +145,7 @@ __device__ __forceinline__ float4 weights4(const TW* w, int d) {
 __device__ __forceinline__ void store4(float* p, const float4 v) { *reinterpret_cast<float4*>(p) = v; }
 __device__ __forceinline__ void store4(bf16_t* p, const float4 v) { *reinterpret_cast<uint2*>(p) = uint2{f32x2_to_bf16x2(v.x, v.y), f32x2_to_bf16x2(v.z, v.w)}; }
 
-template <typename TW, typename TO>
+template <typename TW, typename TO, int NS>
 __global__ __launch_bounds__(256) void streams_norm_shift_fast_kernel(const float* __restrict__ x, long ldx, int n, int width, const float* __restrict__ read,
                                                                      const TW* __restrict__ norm_w, float eps, const float* __restrict__ shift,
                                                                      float* __restrict__ state, long state_stride, const int* __restrict__ pos,
@@ -161,10 +175,10 @@ __global__ __launch_bounds__(256) void streams_norm_shift_fast_kernel(const floa
     for (int i = 0; i < MAXC; ++i) {
         const int d = 4 * (threadIdx.x + 256 * i);
         if (d < width) {
-            u[i] = read_sum4(row, n, width, w, d);
+            u[i] = read_sum4<NS>(row, n, width, w, d);
             ss = squares4(u[i], ss);
             if (both) {
-                ub[i] = read_sum4(row_b, n, width, w, d);
+                ub[i] = read_sum4<NS>(row_b, n, width, w, d);
                 ss_b = squares4(ub[i], ss_b);
             }
         }
@@ -206,7 +220,7 @@ __global__ __launch_bounds__(256) void streams_norm_shift_fast_kernel(const floa
 // x_t <- sum_s mix[s, t] x_s + mult * write[t] * y, and out = norm_w * u / sqrt(mean(u^2) + eps) with u = sum_t read[t] x_t of the new
 // copies.  Up to 8 copies, widths as above.
 constexpr int FUSED_MAX_STREAMS = 8;
-template <typename TW, typename TO>
+template <typename TW, typename TO, int NS>
 __global__ __launch_bounds__(256) void streams_write_norm_kernel(float* __restrict__ x, long ldx, int n, int width, const float* __restrict__ y, long ldy,
                                                                 const float* __restrict__ mix, const float* __restrict__ write, float mult,
                                                                 const float* __restrict__ read, const TW* __restrict__ norm_w, float eps, TO* __restrict__ out, long ldo) {
@@ -228,21 +242,22 @@ __global__ __launch_bounds__(256) void streams_write_norm_kernel(float* __restri
     for (int i = 0; i < MAXC; ++i) {
         const int d = 4 * (threadIdx.x + 256 * i);
         if (d < width) {
-            float4 old[FUSED_MAX_STREAMS];
+            constexpr int MOST = NS > 0 ? NS : FUSED_MAX_STREAMS;          // (NS > 0: the number of copies, known where the kernel is compiled)
+            float4 old[MOST];
 #pragma unroll
-            for (int s = 0; s < FUSED_MAX_STREAMS; ++s)
-                if (s < n) old[s] = ld4(row + (size_t)s * width + d);
+            for (int s = 0; s < MOST; ++s)
+                if (NS > 0 || s < n) old[s] = ld4(row + (size_t)s * width + d);
             const float4 v = ld4(yr + d);
             float4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int to = 0; to < FUSED_MAX_STREAMS; ++to) {
-                if (to < n) {
+            for (int to = 0; to < MOST; ++to) {
+                if (NS > 0 || to < n) {
                     float4 a;
                     if (mix != nullptr) {
                         a = float4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                        for (int s = 0; s < FUSED_MAX_STREAMS; ++s)
-                            if (s < n) {
+                        for (int s = 0; s < MOST; ++s)
+                            if (NS > 0 || s < n) {
                                 const float m = m_s[s * n + to];
                                 a.x = fmaf(m, old[s].x, a.x); a.y = fmaf(m, old[s].y, a.y); a.z = fmaf(m, old[s].z, a.z); a.w = fmaf(m, old[s].w, a.w);
                             }
@@ -346,11 +361,15 @@ GI_API int gi_streams_norm_shift(const float* x, long ldx, int n, int width, con
     // of the two serves is a matter of the sizes alone, so a row's numbers never depend on what else the step holds
     const bool fast = width % 4 == 0 && width <= 1024 * MAXC && ldx % 4 == 0 && ldo % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0 &&
                       (shift == nullptr || (((uintptr_t)shift & 15) == 0 && ((uintptr_t)state & 15) == 0 && state_stride % 4 == 0));
+#define FAST(TW, TO, NS)                                                                                                                                  \
+    streams_norm_shift_fast_kernel<TW, TO, NS><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, read, (const TW*)norm_w, eps, shift, state, state_stride, pos, slot, \
+                                                                           (TO*)out, ldo, n_rows, mode)
 #define LAUNCH(TW, TO)                                                                                                                                    \
     do {                                                                                                                                                  \
-        if (fast)                                                                                                                                         \
-            streams_norm_shift_fast_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, read, (const TW*)norm_w, eps, shift, state, state_stride, pos, \
-                                                                               slot, (TO*)out, ldo, n_rows, mode);                                     \
+        if (fast && n == 1) FAST(TW, TO, 1);                                                                                                              \
+        else if (fast && n == 2) FAST(TW, TO, 2);                                                                                                         \
+        else if (fast && n == 4) FAST(TW, TO, 4);                                                                                                         \
+        else if (fast) FAST(TW, TO, 0);                                                                                                                   \
         else                                                                                                                                              \
             streams_norm_shift_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, read, (const TW*)norm_w, eps, shift, state, state_stride, pos, slot, \
                                                                           (TO*)out, ldo, n_rows, mode);                                                \
@@ -361,6 +380,7 @@ GI_API int gi_streams_norm_shift(const float* x, long ldx, int n, int width, con
     else if (w_dtype == GI_BF16 && out_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
     else return gi_fail("streams_norm_shift: unknown dtypes %d, %d", w_dtype, out_dtype);
 #undef LAUNCH
+#undef FAST
     GI_CHECK_LAUNCH("streams_norm_shift");
     return 0;
 }
@@ -384,13 +404,21 @@ GI_API int gi_streams_write_norm(float* x, long ldx, int n, int width, const flo
                "streams_write_norm: bad sizes (rows %d, %d copies of %d)", n_rows, n, width);
     GI_REQUIRE(ldx % 4 == 0 && ldy % 4 == 0 && ldo % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0 && ((uintptr_t)out & 15) == 0,
                "streams_write_norm: rows must start at multiples of 16 bytes");
-#define LAUNCH(TW, TO) streams_write_norm_kernel<TW, TO><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, y, ldy, mix, write, mult, read, (const TW*)norm_w, eps, (TO*)out, ldo)
+#define GO(TW, TO, NS) streams_write_norm_kernel<TW, TO, NS><<<n_rows, 256, 0, stream>>>(x, ldx, n, width, y, ldy, mix, write, mult, read, (const TW*)norm_w, eps, (TO*)out, ldo)
+#define LAUNCH(TW, TO)                  \
+    do {                                \
+        if (n == 1) GO(TW, TO, 1);      \
+        else if (n == 2) GO(TW, TO, 2); \
+        else if (n == 4) GO(TW, TO, 4); \
+        else GO(TW, TO, 0);             \
+    } while (0)
     if (w_dtype == GI_F32 && out_dtype == GI_F32) LAUNCH(float, float);
     else if (w_dtype == GI_F32 && out_dtype == GI_BF16) LAUNCH(float, bf16_t);
     else if (w_dtype == GI_BF16 && out_dtype == GI_F32) LAUNCH(bf16_t, float);
     else if (w_dtype == GI_BF16 && out_dtype == GI_BF16) LAUNCH(bf16_t, bf16_t);
     else return gi_fail("streams_write_norm: unknown dtypes %d, %d", w_dtype, out_dtype);
 #undef LAUNCH
+#undef GO
     GI_CHECK_LAUNCH("streams_write_norm");
     return 0;
 }
