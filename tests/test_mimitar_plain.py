@@ -185,3 +185,24 @@ def test_what_the_configuration_refuses():
     broken(lambda c: c.pop("norm"))
     broken(lambda c: c.__setitem__("streams", 0))
     broken(lambda c: c.__setitem__("layers", []))
+
+
+def test_a_layer_may_name_a_later_layer_s_weights():
+    import copy
+    from geneinfer_amd.config import parse_config
+    from geneinfer_amd.parts import model_tensor_needs
+    cfg = copy.deepcopy(CONFIGS["A"])
+    cfg["layers"][0]["weights_of"] = 2
+    del cfg["layers"][2]["weights_of"]
+    spec = parse_config(cfg).model_spec()
+    assert [e.layer for e in spec.run_order] == [1, 0, 1, 2, 0]
+    assert {n.name.split(".")[0] for n in model_tensor_needs(spec)} == {"embed", "final", "head", "l1", "l2", "l3"}
+    tokens = [5, 17, 3, 250, 9, 9, 41]
+    w = random_weights(cfg, 6)
+    assert not any(n.startswith("l0.") for n in w)
+    a = P.PlainMimitar(config=cfg, tensors=w).logits(tokens)
+    # the same model with the two entries' places in the file swapped back: layer 0 holds the weights and layer 2 names it
+    back = copy.deepcopy(CONFIGS["A"])
+    w0 = {("l0." + n[3:] if n.startswith("l2.") else n): t for n, t in w.items()}
+    b = P.PlainMimitar(config=back, tensors=w0).logits(tokens)
+    assert torch.equal(a, b)
