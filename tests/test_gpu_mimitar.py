@@ -465,6 +465,28 @@ def test_a_lost_row_before_or_a_shared_slot_shows(folders, tmp_path):
     assert relative_error(a, b) > 0.1
 
 
+def test_layers_in_another_order_and_a_layer_that_names_a_later_one_s_weights(folders, tmp_path):
+    """Configuration A's layers backwards, so that the first layer runs with the weights of the fourth and attention through latents
+    comes before the layer whose weights it uses: order and ownership are the configuration's, nothing of them is fixed."""
+    import copy
+    cfg = copy.deepcopy(CONFIGS["A"])
+    layers = cfg["layers"][::-1]
+    n = len(layers)
+    for l in layers:
+        if "weights_of" in l:
+            l["weights_of"] = n - 1 - l["weights_of"]
+    cfg["layers"] = layers
+    assert [l.get("weights_of") for l in layers] == [3, None, 4, None, None]
+    write_model(tmp_path / "m", cfg, seed=19)
+    own = {"A": tmp_path / "m"}
+    tokens = _prompt(cfg, 50, 14)
+    for dtype in ("float32", "bfloat16"):
+        runner = make_runner(own, "A", dtype)
+        runner.open("r")
+        got = feed(runner, "r", tokens, [13, 2, 20, 1])
+        check_against_plain(own, "A", dtype, tokens, got, f"layers backwards ({dtype})")
+
+
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_greedy_generation_through_the_entry_point_and_the_scheduler(folders, name):
     """Greedy tokens of several prompts, one by one through `LLM.generate` and together through the scheduler (more requests than
