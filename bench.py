@@ -224,7 +224,7 @@ def mimitar_beside_zidevik(args) -> int:
     latents) and the Llama decoder at the same shapes, random weights; measured as `fekorax_beside_llama` measures.  A Mimitar model
     of L layers here carries 4 copies of the residual stream; its layers take turns of four: attention with the Llama layer's heads
     (a norm over the whole query and key projections, a rotation of half of each head with stretched frequencies, scores capped at
-    30) and the Llama layer's feed-forward with clamped halves; the same attention with 8 experts of a quarter of that inner size
+    50) and the Llama layer's feed-forward with clamped halves; the same attention with 8 experts of a quarter of that inner size
     in 4 groups of which 2 are kept, 2 experts a token, and a gated shared expert of half of it; the first layer once more with its
     own cache (no weights of its own); attention through latents (Rigalorn's sizes, a gate per head) with the experts.  Every
     mixer's input is blended with the token before.  One JSON line."""
@@ -253,13 +253,13 @@ def mimitar_beside_zidevik(args) -> int:
                        loop=dict(start=0, stop=min(2, L), times=2), layers=[dict(type="parallel", mixer=mixer, mlp=mlp if i % 2 == 0 else moe) for i in range(L)])
         m_dense = dict(kind="dense", ff=ff, limit=7.0)
         m_moe = dict(kind="moe", router=dict(experts=8, top=2, groups=dict(count=4, keep=2)), expert=dict(ff=ff // 4, limit=7.0), shared=dict(ff=ff // 2, limit=7.0))
-        m_att = dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, softcap=30.0,
-                     rot=dict(dims=hd // 2, base=500000.0, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+        m_att = dict(heads=H, kv_heads=G, dim=hd, vdim=hd, scale=hd ** -0.5, softcap=50.0,
+                     rot=dict(dims=hd // 2, base=500000.0, scaling=dict(factor=32.0, low=1.0, high=4.0, original=8192)))
         m_latent = dict(heads=H, dim=hd, rot_dim=hd // 2, vdim=hd, q_rank=12 * hd, kv_rank=4 * hd, scale=(1.5 * hd) ** -0.5,
-                        rot=dict(dims=hd // 2, base=500000.0, scaling=dict(factor=8.0, original=4096, fast=32.0, slow=1.0)))
+                        rot=dict(dims=hd // 2, base=500000.0, scaling=dict(factor=4.0, original=4096, fast=16.0, slow=2.0)))
         four = lambda i: [dict(type="attention", mixer=m_att, mlp=m_dense), dict(type="attention", mixer=m_att, mlp=m_moe),
                           dict(type="attention", mixer=m_att, mlp=m_dense, weights_of=i), dict(type="latent_attention", mixer=m_latent, mlp=m_moe)]
-        mimitar = dict(architecture="Mimitar", vocab=vocab, width=D, norm=dict(eps=1e-5), streams=4, residual_mult=0.7, logit_scale=0.5, max_positions=T + 1024,
+        mimitar = dict(architecture="Mimitar", vocab=vocab, width=D, norm=dict(eps=1e-5), streams=4, residual_mult=0.5, logit_scale=0.25, max_positions=T + 1024,
                        layers=[l for i in range(0, L, 4) for l in four(i)][:L])
         record["sizes"][size] = {}
         for name, cfg in (("llama", llama), ("rigalorn", rigalorn), ("zidevik", zidevik), ("mimitar", mimitar)):
